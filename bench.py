@@ -1,0 +1,187 @@
+"""Benchmark of the single-GPU MoE MLP hot path on one MI355X.
+
+A step is one forward + backward of ``FMoETransformerMLP`` over one batch of
+synthetic tokens that is already resident in HBM.  The default workload is the
+Mixtral-like layer the target is quoted on (32768 tokens, d_model 4096,
+d_hidden 14336, 8 experts, top-2, bf16, GELU, fused pipeline with 4 chunks).
+
+Prints ONE JSON line with the whole-job tokens/s, a ``roofline`` object for the
+dominant kernel (timed with HIP events on the stream it is launched on, inside
+this script) and a ``cpu_baseline`` object (the brute-force CPU oracle timed on a
+bounded sample of the same workload on the host cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+CONFIGS = {
+    # name: tokens, d_model, d_hidden, experts, top_k, dtype, fused, description
+    "config1": dict(n=4096, d=512, h=1024, e=8, k=2, dtype="f32", fuse=False,
+                    text="config1: 4096 tokens, d512/h1024, 8 experts top-2, fp32 GELU"),
+    "config2": dict(n=16384, d=1024, h=4096, e=16, k=2, dtype="bf16", fuse=False, cap=2458,
+                    text="config2: GShard top-2, 16384 tokens, d1024/h4096, 16 experts, capacity 2458/expert"),
+    "config3": dict(n=16384, d=2048, h=8192, e=64, k=1, dtype="bf16", fuse=False, zipf=1.2,
+                    text="config3: Switch top-1, 16384 tokens, d2048/h8192, 64 experts, Zipf(1.2) routing"),
+    "config4": dict(n=32768, d=4096, h=14336, e=8, k=2, dtype="bf16", fuse=True,
+                    text="config4: Mixtral-like, 32768 tokens, d4096/h14336, 8 experts top-2, bf16 GELU, "
+                         "fused pipeline 4 chunks"),
+    "config5": dict(n=8192, d=2048, h=1024, e=256, k=8, dtype="bf16", fuse=False, ebias=0.5,
+                    text="config5: 8192 tokens, d2048/h1024, 256 experts top-8, biased logits"),
+}
+
+PEAK = {"bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
+HBM_PEAK_GBS = 8000.0
+
+
+def build_layer(cfg, device):
+    import torch
+    import fastermoe_amd as fmoe
+    from fastermoe_amd.gates.base_gate import BaseGate
+    from fastermoe_amd.gates.utils import limit_by_capacity
+
+    dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    n, e, k = cfg["n"], cfg["e"], cfg["k"]
+    gen = torch.Generator().manual_seed(42 + int(cfg["text"][6]))
+    logits = torch.randn(n, e, generator=gen)
+    if "ebias" in cfg:
+        logits = logits + cfg["ebias"] * torch.randn(e, generator=gen)
+    if "zipf" in cfg:
+        p = torch.arange(1, e + 1, dtype=torch.float64) ** -cfg["zipf"]
+        perm = torch.randperm(e, generator=gen)
+        pick = perm[torch.multinomial(p / p.sum(), n, replacement=True, generator=gen)]
+        logits = torch.full((n, e), -10.0).scatter_(1, pick.view(n, 1), 10.0)
+    logits = logits.to(device)
+
+    class SyntheticGate(BaseGate):
+        """Top-k over fixed seeded logits, scores = softmax over the selected logits
+        (unit score for top-1); optional per-expert capacity through the capacity kernels."""
+
+        def __init__(self, d_model, num_expert, world_size, top_k=2):
+            super().__init__(num_expert, world_size)
+            self.top_k = top_k
+
+        def forward(self, inp):
+            val, idx = torch.topk(logits, k=self.top_k, dim=-1)
+            score = torch.softmax(val, dim=-1).to(inp.dtype)
+            if "cap" in cfg:
+                _, _, idx = limit_by_capacity(idx, self.num_expert, 1, cfg["cap"])
+            return idx, score
+
+    layer = fmoe.FMoETransformerMLP(num_expert=e, d_model=cfg["d"], d_hidden=cfg["h"], top_k=k,
+                                    gate=SyntheticGate, activation=torch.nn.GELU())
+    layer.enable_fuse = cfg["fuse"]
+    layer = layer.to(dtype).to(device)
+    gen2 = torch.Generator().manual_seed(7)
+    x = torch.randn(n, cfg["d"], generator=gen2).to(dtype).to(device).requires_grad_(True)
+    grad = torch.randn(n, cfg["d"], generator=gen2).to(dtype).to(device)
+    return layer, x, grad
+
+
+def step(layer, x, grad):
+    layer.zero_grad(set_to_none=True)
+    x.grad = None
+    out = layer(x)
+    out.backward(grad)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="config4", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-steps", type=int, default=3)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures the single-GPU MoE path only; run with --gpus 1 "
+                 "(multi-GPU expert parallelism is not part of it)")
+
+    import torch
+    from fastermoe_amd import _lib
+
+    os.environ.setdefault("FMOE_FUSE_GRAN", "4")
+    cfg = CONFIGS[args.config]
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    device = torch.device("cuda:0")
+    _lib.load()
+    layer, x, grad = build_layer(cfg, device)
+
+    for _ in range(args.warmup):
+        step(layer, x, grad)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(layer, x, grad)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens_per_s = cfg["n"] * args.steps / elapsed
+
+    # per-kernel timing: HIP events recorded by the library on the stream each kernel runs on
+    _lib.profile_enable(True)
+    _lib.profile_collect()
+    for _ in range(args.profile_steps):
+        step(layer, x, grad)
+    prof = _lib.profile_collect()
+    _lib.profile_enable(False)
+
+    kernels = {}
+    for name, (launches, ms, work) in prof.items():
+        if launches == 0:
+            continue
+        is_gemm = name.startswith("gemm")
+        rate = work / (ms * 1e-3) / (1e12 if is_gemm else 1e9)
+        kernels[name] = {"launches_per_step": launches / args.profile_steps,
+                         "avg_ms": ms / launches, "ms_per_step": ms / args.profile_steps,
+                         "work_per_launch": work / launches,
+                         "achieved": rate, "unit": "TFLOP/s" if is_gemm else "GB/s"}
+    gemm_names = [k for k in kernels if k.startswith("gemm")]
+    dominant = max(gemm_names, key=lambda k: kernels[k]["ms_per_step"])
+    peak = PEAK[cfg["dtype"]]
+    dk = kernels[dominant]
+    roofline = {"kernel": "grouped_gemm_kernel (" + dominant + ")", "bound": "mfma", "achieved": round(dk["achieved"], 2),
+                "peak": peak, "unit": "TFLOP/s", "frac": round(dk["achieved"] / peak, 4),
+                "flop_per_launch": dk["work_per_launch"], "avg_launch_ms": round(dk["avg_ms"], 4),
+                "traffic": None}
+    gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_names)
+    gemm_flop = sum(kernels[k]["work_per_launch"] * kernels[k]["launches_per_step"] for k in gemm_names)
+
+    result = {
+        "metric": "moe_mlp_fwd_bwd_tokens_per_s", "value": round(tokens_per_s, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {"workload": cfg["text"], "tokens": cfg["n"], "d_model": cfg["d"], "d_hidden": cfg["h"],
+                   "experts": cfg["e"], "top_k": cfg["k"], "fused": cfg["fuse"],
+                   "chunks": int(os.environ["FMOE_FUSE_GRAN"]) if cfg["fuse"] else 1},
+        "roofline": roofline,
+        "gemm_all": {"tflops": round(gemm_flop / (gemm_ms * 1e-3) / 1e12, 2),
+                     "frac_of_mfma_peak": round(gemm_flop / (gemm_ms * 1e-3) / 1e12 / peak, 4),
+                     "ms_per_step": round(gemm_ms, 3)},
+        "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()}
+                    for k, v in kernels.items()},
+        "hbm_peak_gbs": HBM_PEAK_GBS,
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import moe as omoe
+        sample = {"config1": cfg["n"], "config4": 1024}.get(args.config, 2048)
+        sample = min(sample, cfg["n"])
+        tps, cores, secs = omoe.time_cpu_baseline(sample, cfg["d"], cfg["h"], cfg["e"], cfg["k"], "gelu",
+                                                  seed=1, repeats=1, threads=min(os.cpu_count() or 1, 16))
+        result["cpu_baseline"] = {"value": round(tps, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+                                  "sample": f"{sample} of {cfg['n']} tokens, same d_model/d_hidden/experts/top_k, "
+                                            f"fp32, 1 iteration fwd+bwd, {secs:.1f} s"}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

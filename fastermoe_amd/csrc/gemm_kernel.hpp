@@ -1,0 +1,443 @@
+// Device side of the grouped GEMM: kernel template and its launcher.  Included by
+// gemm_inst.hip (one translation unit per element type and product, so that the
+// variants build in parallel) and by grouped_gemm.hip (host dispatch).
+#pragma once
+#include "grouped_gemm.hpp"
+#include "profile.hpp"
+
+#include <algorithm>
+
+namespace fmoe {
+namespace gemm {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int kSlabBytes = 128;  // contraction bytes per row per slab
+constexpr int kStepsPerSlab = 4; // 32-byte contraction steps (two 16-byte chunks) per slab
+constexpr int kGroupM = 8;       // row tiles that share a column tile consecutively
+
+enum Shape { kKC = 0, kMC = 1 };
+enum Ragged { kRaggedRows = 0, kRaggedK = 1 };
+
+// ---- element traits ---------------------------------------------------------
+template <typename T> struct Elem;
+
+template <> struct Elem<__bf16> {
+    static constexpr int kPerChunk = 8;
+    __device__ static __forceinline__ void mma(f32x16 &acc, const u32x4 &p, const u32x4 &q) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, p), __builtin_bit_cast(bf16x8, q),
+                                                      acc, 0, 0, 0);
+    }
+    __device__ static __forceinline__ float to_float(__bf16 v) { return (float)v; }
+};
+
+template <> struct Elem<_Float16> {
+    static constexpr int kPerChunk = 8;
+    __device__ static __forceinline__ void mma(f32x16 &acc, const u32x4 &p, const u32x4 &q) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, p), __builtin_bit_cast(f16x8, q), acc,
+                                                     0, 0, 0);
+    }
+};
+
+template <> struct Elem<float> {
+    static constexpr int kPerChunk = 4;
+    __device__ static __forceinline__ void mma(f32x16 &acc, const u32x4 &p, const u32x4 &q) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(p[j]), __uint_as_float(q[j]), acc, 0, 0, 0);
+    }
+};
+
+__device__ __forceinline__ float apply_act(float x, int act) {
+    if (act == FMOE_ACT_RELU) return x > 0.f ? x : 0.f;
+    if (act == FMOE_ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
+    return x;
+}
+
+__device__ __forceinline__ float act_grad(float x, int act) {
+    if (act == FMOE_ACT_RELU) return x > 0.f ? 1.f : 0.f;
+    if (act == FMOE_ACT_GELU)
+        return 0.5f * (1.f + erff(x * 0.70710678118654752440f)) + x * 0.39894228040143267794f * __expf(-0.5f * x * x);
+    return 1.f;
+}
+
+// ---- kernel arguments -------------------------------------------------------
+struct GemmParams {
+    const void *P;     // column operand (supplies C's columns)
+    const void *Q;     // row operand (supplies C's rows)
+    void *C;
+    const void *bias;  // per expert [n_cols] or null
+    void *aux;         // see Epilogue
+    int64_t ldp, ldq, ldc;      // leading dimensions in elements
+    int64_t p_expert_stride;    // elements between two experts' P (0: P is row-indexed like Q)
+    int64_t c_expert_stride;    // ragged-K: elements between two experts' C
+    int64_t bias_expert_stride;
+    int32_t n_cols;    // C columns = valid extent of P
+    int32_t n_rows;    // ragged-K: C rows per expert = valid extent of Q
+    int32_t k_extent;  // ragged-rows: contraction length
+    int32_t tiles_n, tiles_m, total_tiles;
+    int32_t activation;
+    int32_t accumulate_first;  // ragged-K: expert 0 of the table adds to C
+    int32_t epilogue;          // Epilogue, read by the any-shape kernel only
+    int32_t profile_class;     // host only: ProfileClass of this launch
+    double profile_work;       // host only: flop of this launch
+    SegmentTable tab;
+};
+
+// KC slabs: 16-byte chunk c of row r is stored at chunk c ^ swz(r).
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+// MC slabs of 16-bit elements: chunk c of contraction row k is stored at c ^ ((k % 4) * 2),
+// so that the four k rows one transposing read touches sit in different banks.
+template <typename T> __device__ __forceinline__ int mc_swz(int k) { return sizeof(T) == 2 ? (k & 3) << 1 : 0; }
+
+// ---- the kernel ---------------------------------------------------------------
+template <typename T, int BM, int BN, int PSHAPE, int QSHAPE, int RAGGED, int EPI>
+__global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
+    constexpr int CE = Elem<T>::kPerChunk;           // elements per 16-byte chunk
+    constexpr int BKE = kSlabBytes / (int)sizeof(T); // elements per slab row
+    constexpr int WM = BM / 2, WN = BN / 2;          // wave tile
+    constexpr int TI = WN / 32, TJ = WM / 32;        // MFMA blocks per wave (cols, rows)
+    constexpr int NP = BN * 8 / kThreads;            // 16-byte chunks per thread per slab
+    constexpr int NQ = BM * 8 / kThreads;
+    constexpr int P_BYTES = BN * kSlabBytes, Q_BYTES = BM * kSlabBytes;
+    constexpr int STAGE_BYTES = P_BYTES + Q_BYTES;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    // -- which tile ------------------------------------------------------------
+    const int per_xcd = (gridDim.x + 7) >> 3;
+    const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (L >= prm.total_tiles) return;
+
+    int ei, mt, nt;
+    {
+        int tm_total, rem;
+        if (RAGGED == kRaggedRows) {
+            tm_total = prm.tab.tile[prm.tab.n];
+            rem = L;
+            ei = 0;
+        } else {
+            const int tpe = prm.tiles_m * prm.tiles_n;
+            tm_total = prm.tiles_m;
+            ei = L / tpe;
+            rem = L - ei * tpe;
+        }
+        const int gspan = kGroupM * prm.tiles_n;
+        const int grp = rem / gspan;
+        const int first_m = grp * kGroupM;
+        const int gsz = min(kGroupM, tm_total - first_m);
+        const int in_grp = rem - grp * gspan;
+        mt = first_m + in_grp % gsz;
+        nt = in_grp / gsz;
+        if (RAGGED == kRaggedRows) {
+            int lo = 0, hi = prm.tab.n;  // tile[lo] <= mt < tile[hi]
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (prm.tab.tile[mid] <= mt) lo = mid; else hi = mid;
+            }
+            ei = lo;
+        }
+    }
+    const int expert = prm.tab.first_expert + ei;
+    const int seg_lo = prm.tab.seg[ei], seg_hi = prm.tab.seg[ei + 1];
+    const int n0 = nt * BN;
+
+    const T *Pb;
+    const T *Qb;
+    T *Cb;
+    int p_valid, q_valid, K;
+    int64_t aux_off;  // offset of this tile's origin inside C (and aux)
+    if (RAGGED == kRaggedRows) {
+        const int row0 = seg_lo + (mt - prm.tab.tile[ei]) * BM;
+        q_valid = min(BM, seg_hi - row0);
+        K = prm.k_extent;
+        Qb = (const T *)prm.Q + (int64_t)row0 * prm.ldq;
+        const T *Pe = (const T *)prm.P + (int64_t)expert * prm.p_expert_stride;
+        Pb = (PSHAPE == kKC) ? Pe + (int64_t)n0 * prm.ldp : Pe + n0;
+        aux_off = (int64_t)row0 * prm.ldc + n0;
+    } else {
+        const int m0 = mt * BM;
+        q_valid = min(BM, prm.n_rows - m0);
+        K = seg_hi - seg_lo;
+        Qb = (const T *)prm.Q + (int64_t)seg_lo * prm.ldq + m0;
+        Pb = (const T *)prm.P + (int64_t)seg_lo * prm.ldp + n0;
+        aux_off = (int64_t)expert * prm.c_expert_stride + (int64_t)m0 * prm.ldc + n0;
+    }
+    p_valid = min(BN, prm.n_cols - n0);
+    Cb = (T *)prm.C + aux_off;
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int wave_m0 = (wave >> 1) * WM, wave_n0 = (wave & 1) * WN;
+
+    // -- global -> register -> LDS staging ---------------------------------------
+    // KC: chunk q = it*256 + t covers row q/8, chunk q%8 of the slab.
+    // MC: chunk q covers contraction row q / CPR, 16-byte column chunk q % CPR.
+    u32x4 pg[NP], qg[NQ];
+
+    auto load_slab = [&](int k0) {
+        if (PSHAPE == kKC) {
+            const int r_t = t >> 3, c_t = t & 7;
+            const bool kok = k0 + c_t * CE < K;
+            const T *src = Pb + (int64_t)r_t * prm.ldp + k0 + c_t * CE;
+#pragma unroll
+            for (int it = 0; it < NP; ++it) {
+                pg[it] = u32x4{0, 0, 0, 0};
+                if (kok && it * 32 + r_t < p_valid) pg[it] = *(const u32x4 *)(src + (int64_t)it * 32 * prm.ldp);
+            }
+        } else {
+            constexpr int CPR = BN / CE, KPI = kThreads / CPR;
+            const int kk_t = t / CPR, c_t = t % CPR;
+            const bool rok = c_t * CE < p_valid;
+            const T *src = Pb + (int64_t)(k0 + kk_t) * prm.ldp + c_t * CE;
+#pragma unroll
+            for (int it = 0; it < NP; ++it) {
+                pg[it] = u32x4{0, 0, 0, 0};
+                if (rok && k0 + kk_t + it * KPI < K) pg[it] = *(const u32x4 *)(src + (int64_t)it * KPI * prm.ldp);
+            }
+        }
+        if (QSHAPE == kKC) {
+            const int r_t = t >> 3, c_t = t & 7;
+            const bool kok = k0 + c_t * CE < K;
+            const T *src = Qb + (int64_t)r_t * prm.ldq + k0 + c_t * CE;
+#pragma unroll
+            for (int it = 0; it < NQ; ++it) {
+                qg[it] = u32x4{0, 0, 0, 0};
+                if (kok && it * 32 + r_t < q_valid) qg[it] = *(const u32x4 *)(src + (int64_t)it * 32 * prm.ldq);
+            }
+        } else {
+            constexpr int CPR = BM / CE, KPI = kThreads / CPR;
+            const int kk_t = t / CPR, c_t = t % CPR;
+            const bool rok = c_t * CE < q_valid;
+            const T *src = Qb + (int64_t)(k0 + kk_t) * prm.ldq + c_t * CE;
+#pragma unroll
+            for (int it = 0; it < NQ; ++it) {
+                qg[it] = u32x4{0, 0, 0, 0};
+                if (rok && k0 + kk_t + it * KPI < K) qg[it] = *(const u32x4 *)(src + (int64_t)it * KPI * prm.ldq);
+            }
+        }
+    };
+
+    auto store_slab = [&](int stage) {
+        unsigned char *sp = smem + stage * STAGE_BYTES;
+        unsigned char *sq = sp + P_BYTES;
+        if (PSHAPE == kKC) {
+            const int r_t = t >> 3, c_t = t & 7;
+            const int off = r_t * kSlabBytes + ((c_t ^ swz(r_t)) << 4);
+#pragma unroll
+            for (int it = 0; it < NP; ++it) *(u32x4 *)(sp + off + it * 32 * kSlabBytes) = pg[it];
+        } else {
+            constexpr int CPR = BN / CE, KPI = kThreads / CPR;
+            const int kk_t = t / CPR, c_t = t % CPR;
+#pragma unroll
+            for (int it = 0; it < NP; ++it) {
+                const int kk = kk_t + it * KPI;
+                *(u32x4 *)(sp + (kk * CPR + (c_t ^ mc_swz<T>(kk))) * 16) = pg[it];
+            }
+        }
+        if (QSHAPE == kKC) {
+            const int r_t = t >> 3, c_t = t & 7;
+            const int off = r_t * kSlabBytes + ((c_t ^ swz(r_t)) << 4);
+#pragma unroll
+            for (int it = 0; it < NQ; ++it) *(u32x4 *)(sq + off + it * 32 * kSlabBytes) = qg[it];
+        } else {
+            constexpr int CPR = BM / CE, KPI = kThreads / CPR;
+            const int kk_t = t / CPR, c_t = t % CPR;
+#pragma unroll
+            for (int it = 0; it < NQ; ++it) {
+                const int kk = kk_t + it * KPI;
+                *(u32x4 *)(sq + (kk * CPR + (c_t ^ mc_swz<T>(kk))) * 16) = qg[it];
+            }
+        }
+    };
+
+    // -- fragments ---------------------------------------------------------------
+    // A fragment is the 16 bytes a lane feeds to the MFMA for one 32-row block and
+    // one contraction step: row = block row l32, contraction chunk = 2*step + h.
+    auto frag = [&](const unsigned char *slab, int shape, int extent, int r0, int ks) -> u32x4 {
+        const int row = r0 + l32;
+        if (shape == kKC) {
+            const int chunk = ks * 2 + h;
+            return *(const u32x4 *)(slab + row * kSlabBytes + ((chunk ^ swz(row)) << 4));
+        }
+        u32x4 out;
+        if (sizeof(T) == 4) {
+            const uint32_t *s = (const uint32_t *)slab;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) out[j] = s[(ks * 8 + h * 4 + j) * extent + row];
+        } else {
+            // ds_read_b64_tr_b16: a 16-lane group reads a 4(k) x 16(row) block of 16-bit
+            // elements, lane s of the group pointing at row-of-k s/4, columns 4*(s%4)..+3,
+            // and receives column s of the block with its 4 k values.  Groups 0/1 take rows
+            // 0-15/16-31 of the 32-row block, groups 2/3 the same rows 8 k further on.
+            const int grp = lane >> 4, s16 = lane & 15;
+            const int col = r0 + (grp & 1) * 16 + 4 * (s16 & 3);
+            const int kq = s16 >> 2;
+            const int chunk = (col >> 3) ^ (kq << 1);   // MC slabs are swizzled by k % 4
+            const int kb = ks * 16 + (grp >> 1) * 8 + kq;
+            const unsigned char *base = slab + chunk * 16 + (col & 7) * 2;
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_ptr;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(base + kb * extent * 2));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(base + (kb + 4) * extent * 2));
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            out = u32x4{l2[0], l2[1], h2[0], h2[1]};
+        }
+        return out;
+    };
+
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int x = 0; x < TI; ++x)
+#pragma unroll
+        for (int y = 0; y < TJ; ++y)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[x][y][r] = 0.f;
+
+    const int n_slabs = (K + BKE - 1) / BKE;
+    if (n_slabs > 0) {
+        load_slab(0);
+        store_slab(0);
+    }
+    __syncthreads();
+    for (int s = 0; s < n_slabs; ++s) {
+        if (s + 1 < n_slabs) load_slab((s + 1) * BKE);
+        const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
+        const unsigned char *sq = sp + P_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < kStepsPerSlab; ++ks) {
+            u32x4 pf[TI], qf[TJ];
+#pragma unroll
+            for (int x = 0; x < TI; ++x) pf[x] = frag(sp, PSHAPE, BN, wave_n0 + x * 32, ks);
+#pragma unroll
+            for (int y = 0; y < TJ; ++y) qf[y] = frag(sq, QSHAPE, BM, wave_m0 + y * 32, ks);
+#pragma unroll
+            for (int x = 0; x < TI; ++x)
+#pragma unroll
+                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[x], qf[y]);
+        }
+        if (s + 1 < n_slabs) store_slab((s + 1) & 1);
+        __syncthreads();
+    }
+
+    // -- epilogue ------------------------------------------------------------------
+    // acc[x][y][4*g + i] is C(row = wave_m0 + 32*y + l32, col = wave_n0 + 32*x + 8*g + 4*h + i).
+    const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride + n0 : nullptr;
+    T *aux = prm.aux ? (T *)prm.aux + aux_off : nullptr;
+    const bool accumulate = (RAGGED == kRaggedK) && prm.accumulate_first && ei == 0;
+#pragma unroll
+    for (int y = 0; y < TJ; ++y) {
+        const int row = wave_m0 + y * 32 + l32;
+        if (row >= q_valid) continue;
+#pragma unroll
+        for (int x = 0; x < TI; ++x) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int col = wave_n0 + x * 32 + g * 8 + h * 4;
+                if (col >= p_valid) continue;
+                float v[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = acc[x][y][4 * g + i];
+                T *dst = Cb + (int64_t)row * prm.ldc + col;
+                if (bias) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] += (float)bias[col + i];
+                }
+                if (EPI == kEpiBiasAct) {
+                    if (aux) {
+                        alignas(16) T pre[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) pre[i] = (T)v[i];
+                        T *adst = aux + (int64_t)row * prm.ldc + col;
+                        if (sizeof(T) == 2) *(u32x2 *)adst = *(const u32x2 *)pre;
+                        else *(u32x4 *)adst = *(const u32x4 *)pre;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = apply_act(v[i], prm.activation);
+                } else if (EPI == kEpiDAct) {
+                    alignas(16) T pre[4];
+                    const T *asrc = aux + (int64_t)row * prm.ldc + col;
+                    if (sizeof(T) == 2) *(u32x2 *)pre = *(const u32x2 *)asrc;
+                    else *(u32x4 *)pre = *(const u32x4 *)asrc;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] *= act_grad((float)pre[i], prm.activation);
+                }
+                if (accumulate) {
+                    alignas(16) T old[4];
+                    if (sizeof(T) == 2) *(u32x2 *)old = *(const u32x2 *)dst;
+                    else *(u32x4 *)old = *(const u32x4 *)dst;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] += (float)old[i];
+                }
+                alignas(16) T res[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) res[i] = (T)v[i];
+                if (sizeof(T) == 2) *(u32x2 *)dst = *(const u32x2 *)res;
+                else *(u32x4 *)dst = *(const u32x4 *)res;
+            }
+        }
+    }
+}
+
+template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI>
+int launch_tiles(GemmParams &prm, hipStream_t stream) {
+    constexpr int smem = 2 * (BM + BN) * kSlabBytes;
+    static bool configured = false;
+    auto kern = grouped_gemm_kernel<T, BM, BN, PS, QS, RG, EPI>;
+    if (!configured) {
+        FMOE_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        configured = true;
+    }
+    if (prm.total_tiles <= 0) return FMOE_OK;
+    const int grid = (prm.total_tiles + 7) / 8 * 8;
+    ProfileScope prof(prm.profile_class, prm.profile_work, stream);
+    kern<<<grid, kThreads, smem, stream>>>(prm);
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+// Tile counts for a 256 x 256 tiling, then the launch for the requested epilogue.
+// EPI_MASK lists the epilogues a product can be asked for, so that only those
+// kernels are built.
+template <typename T, int PS, int QS, int RG, int EPI_MASK>
+int launch_by_epilogue(GemmParams &prm, int epi, hipStream_t stream) {
+    constexpr int BM = 256, BN = 256;
+    prm.tiles_n = (int)ceil_div(prm.n_cols, BN);
+    if (RG == kRaggedRows) {
+        prm.tiles_m = 0;
+        prm.total_tiles = prm.tab.tile[prm.tab.n] * prm.tiles_n;
+    } else {
+        prm.tiles_m = (int)ceil_div(prm.n_rows, BM);
+        prm.total_tiles = prm.tab.n * prm.tiles_m * prm.tiles_n;
+    }
+    if constexpr ((EPI_MASK >> kEpiStore) & 1)
+        if (epi == kEpiStore) return launch_tiles<T, BM, BN, PS, QS, RG, kEpiStore>(prm, stream);
+    if constexpr ((EPI_MASK >> kEpiBiasAct) & 1)
+        if (epi == kEpiBiasAct) return launch_tiles<T, BM, BN, PS, QS, RG, kEpiBiasAct>(prm, stream);
+    if constexpr ((EPI_MASK >> kEpiDAct) & 1)
+        if (epi == kEpiDAct) return launch_tiles<T, BM, BN, PS, QS, RG, kEpiDAct>(prm, stream);
+    return fail(FMOE_EINVAL, "epilogue %d is not built for this product", epi);
+}
+
+}  // namespace gemm
+
+// Defined in gemm_inst.hip, once per (element type, product).
+#define FMOE_DECLARE_MFMA(NAME) int NAME(gemm::GemmParams &prm, int epilogue, hipStream_t stream)
+FMOE_DECLARE_MFMA(launch_mfma_bf16_fwd);
+FMOE_DECLARE_MFMA(launch_mfma_bf16_dgrad);
+FMOE_DECLARE_MFMA(launch_mfma_bf16_wgrad);
+FMOE_DECLARE_MFMA(launch_mfma_f16_fwd);
+FMOE_DECLARE_MFMA(launch_mfma_f16_dgrad);
+FMOE_DECLARE_MFMA(launch_mfma_f16_wgrad);
+FMOE_DECLARE_MFMA(launch_mfma_f32_fwd);
+FMOE_DECLARE_MFMA(launch_mfma_f32_dgrad);
+FMOE_DECLARE_MFMA(launch_mfma_f32_wgrad);
+
+}  // namespace fmoe

@@ -1,0 +1,395 @@
+// Grouped GEMM over ragged expert segments for gfx950 (MI355X, CDNA4).
+//
+// One launch covers every expert: the row segments travel in the kernel
+// arguments, a workgroup finds its (expert, row tile, column tile) by a binary
+// search over the tile prefix, and there is no per-expert launch, no host loop
+// over streams and no host synchronisation.
+//
+// Three products share one kernel template:
+//   forward  Y[seg]  = X[seg] . W_e^T      rows ragged, contraction = in
+//   dgrad    dX[seg] = dY[seg] . W_e       rows ragged, contraction = out
+//   wgrad    dW_e    = dY[seg]^T . X[seg]  contraction ragged (the segment)
+//
+// Tiling.  A 256-thread workgroup (4 waves, 2 x 2) owns a BM x BN tile of C and
+// walks the contraction in slabs of 128 bytes per row (64 bf16 / 32 fp32).
+// Both operand slabs are staged in LDS, double buffered: the global loads of
+// slab k+1 are issued before the MFMAs of slab k and written to the other LDS
+// buffer afterwards, one barrier per slab.  Each wave computes a
+// (BM/2) x (BN/2) sub-tile as 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16 /
+// _f16, v_mfma_f32_32x32x2_f32), accumulating in fp32.
+//
+// The MFMA's row index is mapped to C's COLUMN, so a lane ends up with four
+// consecutive columns of one row in adjacent accumulator registers and the
+// epilogue stores them as one 8/16-byte vector.
+//
+// Operands come in two memory shapes.  "KC": the contraction index is the
+// contiguous one (X, dY as the row operand, W in forward); the LDS slab is
+// [row][128 B] with the 16-byte chunks XOR-swizzled by the row so that the
+// 16-byte fragment reads of 32 consecutive rows spread over all banks.  "MC":
+// the row index is contiguous and the contraction strided (W in dgrad, both
+// operands in wgrad); the slab is kept as [k][rows] and the fragment is
+// collected along k when it is read.
+#include "gemm_kernel.hpp"
+#include "profile.hpp"
+
+#include <algorithm>
+#include <initializer_list>
+
+namespace fmoe {
+using namespace gemm;
+namespace {
+
+// ---- any-shape fallback (odd feature sizes, fp64): one thread per C element ----
+template <typename T, typename Acc, int RAGGED, int PSHAPE>
+__global__ __launch_bounds__(kThreads) void grouped_gemm_plain_kernel(const GemmParams prm) {
+    const int ei = blockIdx.z;
+    const int expert = prm.tab.first_expert + ei;
+    const int seg_lo = prm.tab.seg[ei], seg_hi = prm.tab.seg[ei + 1];
+    const int col = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int rows = (RAGGED == kRaggedRows) ? seg_hi - seg_lo : prm.n_rows;
+    const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride : nullptr;
+    const bool accumulate = (RAGGED == kRaggedK) && prm.accumulate_first && ei == 0;
+    if (col >= prm.n_cols) return;
+    for (int row = blockIdx.y * 16 + (threadIdx.x >> 4); row < rows; row += gridDim.y * 16) {
+        Acc acc = 0;
+        int64_t c_off;
+        if (RAGGED == kRaggedRows) {
+            const T *q = (const T *)prm.Q + (int64_t)(seg_lo + row) * prm.ldq;
+            const T *p = (const T *)prm.P + (int64_t)expert * prm.p_expert_stride;
+            for (int k = 0; k < prm.k_extent; ++k) {
+                const Acc pv = (PSHAPE == kKC) ? (Acc)p[(int64_t)col * prm.ldp + k] : (Acc)p[(int64_t)k * prm.ldp + col];
+                acc += (Acc)q[k] * pv;
+            }
+            c_off = (int64_t)(seg_lo + row) * prm.ldc + col;
+        } else {
+            const T *q = (const T *)prm.Q + (int64_t)seg_lo * prm.ldq + row;
+            const T *p = (const T *)prm.P + (int64_t)seg_lo * prm.ldp + col;
+            for (int k = 0; k < seg_hi - seg_lo; ++k) acc += (Acc)q[(int64_t)k * prm.ldq] * (Acc)p[(int64_t)k * prm.ldp];
+            c_off = (int64_t)expert * prm.c_expert_stride + (int64_t)row * prm.ldc + col;
+        }
+        T *dst = (T *)prm.C + c_off;
+        if (bias) acc += (Acc)bias[col];
+        if (prm.epilogue == kEpiBiasAct) {
+            if (prm.aux) ((T *)prm.aux)[c_off] = (T)acc;
+            acc = (Acc)apply_act((float)acc, prm.activation);
+        } else if (prm.epilogue == kEpiDAct) {
+            acc *= (Acc)act_grad((float)((const T *)prm.aux)[c_off], prm.activation);
+        }
+        if (accumulate) acc += (Acc)*dst;
+        *dst = (T)acc;
+    }
+}
+
+// ---- bias gradient: column sums per expert segment ---------------------------------
+// Thread (c, g) adds rows g, g+4, ... of column c in order; the four partial sums
+// are then added in a fixed order, so the result is reproducible.
+template <typename T, typename Acc>
+__global__ __launch_bounds__(kThreads) void bias_grad_kernel(const T *__restrict__ gy, T *__restrict__ gb,
+                                                             int64_t out_feat, const SegmentTable tab,
+                                                             int accumulate_first) {
+    __shared__ Acc part[4][64];
+    const int ei = blockIdx.y;
+    const int expert = tab.first_expert + ei;
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int g = threadIdx.x >> 6;
+    Acc acc = 0;
+    if (c < out_feat)
+        for (int r = tab.seg[ei] + g; r < tab.seg[ei + 1]; r += 4) acc += (Acc)gy[(int64_t)r * out_feat + c];
+    part[g][threadIdx.x & 63] = acc;
+    __syncthreads();
+    if (g == 0 && c < out_feat) {
+        Acc s = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) + part[3][threadIdx.x];
+        T *dst = gb + (int64_t)expert * out_feat + c;
+        if (accumulate_first && ei == 0) s += (Acc)*dst;
+        *dst = (T)s;
+    }
+}
+
+// ---- host side ---------------------------------------------------------------------------
+
+struct Plan {
+    int first, last;       // experts [first, last] covered (last < first: nothing)
+    bool accumulate_first; // the first covered expert began before row_lo
+};
+
+// Row segments of experts [e0, e1] clipped to [row_lo, row_hi): seg[i] is the
+// clipped start of expert e0+i, seg[n] the clipped end of expert e1.
+void fill_table(SegmentTable *tab, const int64_t *counts, int e0, int e1, int64_t row_lo, int64_t row_hi,
+                int block_rows) {
+    auto clip = [&](int64_t r) { return r < row_lo ? row_lo : (r > row_hi ? row_hi : r); };
+    int64_t start = 0;
+    for (int e = 0; e < e0; ++e) start += counts[e];
+    tab->n = e1 - e0 + 1;
+    tab->first_expert = e0;
+    int tiles = 0;
+    for (int e = e0; e <= e1; ++e) {
+        const int64_t end = start + counts[e];
+        const int64_t lo = clip(start), hi = clip(end);
+        tab->seg[e - e0] = (int32_t)lo;
+        tab->seg[e - e0 + 1] = (int32_t)hi;
+        tab->tile[e - e0] = tiles;
+        tiles += (int)ceil_div(hi - lo, block_rows);
+        start = end;
+    }
+    tab->tile[tab->n] = tiles;
+}
+
+double table_flop(const SegmentTable &tab, int64_t in_feat, int64_t out_feat) {
+    return 2.0 * (double)(tab.seg[tab.n] - tab.seg[0]) * (double)in_feat * (double)out_feat;
+}
+
+int check_counts(const char *who, const int64_t *counts, int64_t n_expert, int64_t row_lo, int64_t row_hi,
+                 int64_t *total) {
+    FMOE_REQUIRE(counts != nullptr, "%s: expert_count_host is NULL", who);
+    FMOE_REQUIRE(n_expert >= 1, "%s: n_expert=%lld", who, (long long)n_expert);
+    int64_t s = 0;
+    for (int64_t e = 0; e < n_expert; ++e) {
+        FMOE_REQUIRE(counts[e] >= 0, "%s: expert_count[%lld]=%lld is negative", who, (long long)e,
+                     (long long)counts[e]);
+        s += counts[e];
+    }
+    if (s > (int64_t)INT32_MAX || n_expert > (int64_t)(1 << 24))
+        return fail(FMOE_ELIMIT, "%s: %lld rows / %lld experts exceed the supported range", who, (long long)s,
+                    (long long)n_expert);
+    FMOE_REQUIRE(row_lo >= 0 && row_lo <= row_hi && row_hi <= s, "%s: row range [%lld,%lld) outside [0,%lld]", who,
+                 (long long)row_lo, (long long)row_hi, (long long)s);
+    *total = s;
+    return FMOE_OK;
+}
+
+// experts that own at least one row of [row_lo, row_hi)
+Plan plan_rows(const int64_t *counts, int64_t n_expert, int64_t row_lo, int64_t row_hi) {
+    Plan p{0, -1, false};
+    int64_t start = 0;
+    bool any = false;
+    for (int e = 0; e < (int)n_expert; ++e) {
+        const int64_t end = start + counts[e];
+        if (end > row_lo && start < row_hi && end > start) {
+            if (!any) { p.first = e; p.accumulate_first = start < row_lo; any = true; }
+            p.last = e;
+        }
+        start = end;
+    }
+    return p;
+}
+
+// experts this chunk must WRITE in a ragged-K product: those with rows in the
+// chunk, plus row-less experts positioned inside it.
+Plan plan_contraction(const int64_t *counts, int64_t n_expert, int64_t row_lo, int64_t row_hi, bool last_chunk) {
+    Plan p{0, -1, false};
+    int64_t start = 0;
+    bool any = false;
+    for (int e = 0; e < (int)n_expert; ++e) {
+        const int64_t end = start + counts[e];
+        const bool has_rows = end > start && end > row_lo && start < row_hi;
+        const bool empty_here = end == start && ((start >= row_lo && start < row_hi) || (last_chunk && start == row_hi));
+        if (has_rows || empty_here) {
+            if (!any) { p.first = e; p.accumulate_first = has_rows && start < row_lo; any = true; }
+            p.last = e;
+        }
+        start = end;
+    }
+    return p;
+}
+
+template <typename T> bool fast_ok(std::initializer_list<const void *> ptrs, std::initializer_list<int64_t> dims) {
+    constexpr int CE = 16 / (int)sizeof(T);
+    for (const void *p : ptrs)
+        if (p && !aligned16(p)) return false;
+    for (int64_t d : dims)
+        if (d % CE != 0) return false;
+    return true;
+}
+
+template <typename T, typename Acc, int RG, int PS>
+int launch_plain(GemmParams &prm, int epi, hipStream_t stream) {
+    prm.epilogue = epi;
+    int max_rows = 0;
+    if (RG == kRaggedRows) {
+        for (int i = 0; i < prm.tab.n; ++i) max_rows = std::max(max_rows, prm.tab.seg[i + 1] - prm.tab.seg[i]);
+    } else {
+        max_rows = prm.n_rows;
+    }
+    if (max_rows == 0 || prm.n_cols == 0) return FMOE_OK;
+    dim3 grid((unsigned)ceil_div(prm.n_cols, 16), (unsigned)std::min<int64_t>(ceil_div(max_rows, 16), 1024),
+              (unsigned)prm.tab.n);
+    ProfileScope prof(prm.profile_class, prm.profile_work, stream);
+    grouped_gemm_plain_kernel<T, Acc, RG, PS><<<grid, kThreads, 0, stream>>>(prm);
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+enum Product { kFwd = 0, kDgrad = 1, kWgrad = 2 };
+
+template <int PRODUCT>
+int dispatch(GemmParams &prm, int dtype, int epi, bool fast, hipStream_t stream) {
+    constexpr int RG = PRODUCT == kWgrad ? kRaggedK : kRaggedRows;
+    constexpr int PS = PRODUCT == kFwd ? kKC : kMC;
+    if (!fast || dtype == FMOE_F64) {
+        switch (dtype) {
+            case FMOE_BF16: return launch_plain<__bf16, float, RG, PS>(prm, epi, stream);
+            case FMOE_F16: return launch_plain<_Float16, float, RG, PS>(prm, epi, stream);
+            case FMOE_F32: return launch_plain<float, float, RG, PS>(prm, epi, stream);
+            case FMOE_F64: return launch_plain<double, double, RG, PS>(prm, epi, stream);
+        }
+        return fail(FMOE_EINVAL, "unknown dtype %d", dtype);
+    }
+    switch (dtype * 3 + PRODUCT) {
+        case FMOE_BF16 * 3 + kFwd: return launch_mfma_bf16_fwd(prm, epi, stream);
+        case FMOE_BF16 * 3 + kDgrad: return launch_mfma_bf16_dgrad(prm, epi, stream);
+        case FMOE_BF16 * 3 + kWgrad: return launch_mfma_bf16_wgrad(prm, epi, stream);
+        case FMOE_F16 * 3 + kFwd: return launch_mfma_f16_fwd(prm, epi, stream);
+        case FMOE_F16 * 3 + kDgrad: return launch_mfma_f16_dgrad(prm, epi, stream);
+        case FMOE_F16 * 3 + kWgrad: return launch_mfma_f16_wgrad(prm, epi, stream);
+        case FMOE_F32 * 3 + kFwd: return launch_mfma_f32_fwd(prm, epi, stream);
+        case FMOE_F32 * 3 + kDgrad: return launch_mfma_f32_dgrad(prm, epi, stream);
+        case FMOE_F32 * 3 + kWgrad: return launch_mfma_f32_wgrad(prm, epi, stream);
+    }
+    return fail(FMOE_EINVAL, "unknown dtype %d", dtype);
+}
+
+bool is_fast(int dtype, std::initializer_list<const void *> ptrs, std::initializer_list<int64_t> dims) {
+    switch (dtype) {
+        case FMOE_BF16: return fast_ok<__bf16>(ptrs, dims);
+        case FMOE_F16: return fast_ok<_Float16>(ptrs, dims);
+        case FMOE_F32: return fast_ok<float>(ptrs, dims);
+    }
+    return false;
+}
+
+}  // namespace
+
+int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
+                           int64_t row_hi, hipStream_t stream) {
+    int64_t total;
+    if (int rc = check_counts("linear_forward", counts, n_expert, row_lo, row_hi, &total)) return rc;
+    FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
+                 "linear_forward: in_feat=%lld out_feat=%lld", (long long)a.in_feat, (long long)a.out_feat);
+    if (row_hi == row_lo) return FMOE_OK;
+    FMOE_REQUIRE(a.x && a.w && a.y, "linear_forward: NULL tensor");
+    const Plan plan = plan_rows(counts, n_expert, row_lo, row_hi);
+    const bool fast = is_fast(a.dtype, {a.x, a.w, a.y, a.aux, a.bias}, {a.in_feat, a.out_feat});
+    for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
+        const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
+        GemmParams prm{};
+        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, 256);
+        prm.profile_class = kProfGemmFwd; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
+        prm.P = a.w; prm.Q = a.x; prm.C = a.y; prm.bias = a.bias; prm.aux = a.aux;
+        prm.ldp = a.in_feat; prm.ldq = a.in_feat; prm.ldc = a.out_feat;
+        prm.p_expert_stride = a.in_feat * a.out_feat;
+        prm.bias_expert_stride = a.out_feat;
+        prm.n_cols = (int)a.out_feat; prm.k_extent = (int)a.in_feat;
+        prm.activation = a.activation;
+        if (int rc = dispatch<kFwd>(prm, a.dtype, a.epilogue, fast, stream)) return rc;
+    }
+    return FMOE_OK;
+}
+
+int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
+                         int64_t row_hi, hipStream_t stream) {
+    int64_t total;
+    if (int rc = check_counts("linear_dgrad", counts, n_expert, row_lo, row_hi, &total)) return rc;
+    FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
+                 "linear_dgrad: in_feat=%lld out_feat=%lld", (long long)a.in_feat, (long long)a.out_feat);
+    if (row_hi == row_lo) return FMOE_OK;
+    FMOE_REQUIRE(a.gy && a.w && a.gx, "linear_dgrad: NULL tensor");
+    const Plan plan = plan_rows(counts, n_expert, row_lo, row_hi);
+    const bool fast = is_fast(a.dtype, {a.gy, a.w, a.gx, a.aux}, {a.in_feat, a.out_feat});
+    for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
+        const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
+        GemmParams prm{};
+        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, 256);
+        prm.profile_class = kProfGemmDgrad; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
+        prm.P = a.w; prm.Q = a.gy; prm.C = a.gx; prm.aux = const_cast<void *>(a.aux);
+        prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
+        prm.p_expert_stride = a.in_feat * a.out_feat;
+        prm.n_cols = (int)a.in_feat; prm.k_extent = (int)a.out_feat;
+        prm.activation = a.activation;
+        if (int rc = dispatch<kDgrad>(prm, a.dtype, a.epilogue, fast, stream)) return rc;
+    }
+    return FMOE_OK;
+}
+
+int grouped_linear_wgrad(const LinearWgradArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
+                         int64_t row_hi, bool last_chunk, hipStream_t stream) {
+    int64_t total;
+    if (int rc = check_counts("linear_wgrad", counts, n_expert, row_lo, row_hi, &total)) return rc;
+    FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
+                 "linear_wgrad: in_feat=%lld out_feat=%lld", (long long)a.in_feat, (long long)a.out_feat);
+    FMOE_REQUIRE(a.gw && (total == 0 || (a.gy && a.x)), "linear_wgrad: NULL tensor");
+    const Plan plan = plan_contraction(counts, n_expert, row_lo, row_hi, last_chunk);
+    const bool fast = is_fast(a.dtype, {a.gy, a.x, a.gw}, {a.in_feat, a.out_feat});
+    for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
+        const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
+        GemmParams prm{};
+        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, 256);
+        prm.profile_class = kProfGemmWgrad; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
+        prm.P = a.x; prm.Q = a.gy; prm.C = a.gw;
+        prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
+        prm.c_expert_stride = a.in_feat * a.out_feat;
+        prm.n_cols = (int)a.in_feat; prm.n_rows = (int)a.out_feat;
+        prm.accumulate_first = (e0 == plan.first && plan.accumulate_first) ? 1 : 0;
+        if (int rc = dispatch<kWgrad>(prm, a.dtype, kEpiStore, fast, stream)) return rc;
+    }
+    return FMOE_OK;
+}
+
+int grouped_bias_grad(const void *gy, void *gb, int64_t out_feat, int dtype, const int64_t *counts,
+                      int64_t n_expert, int64_t row_lo, int64_t row_hi, bool last_chunk, hipStream_t stream) {
+    int64_t total;
+    if (int rc = check_counts("bias_grad", counts, n_expert, row_lo, row_hi, &total)) return rc;
+    FMOE_REQUIRE(gb && (total == 0 || gy) && out_feat >= 1, "bias_grad: bad argument");
+    const Plan plan = plan_contraction(counts, n_expert, row_lo, row_hi, last_chunk);
+    for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
+        const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
+        SegmentTable tab;
+        fill_table(&tab, counts, e0, e1, row_lo, row_hi, 256);
+        const int acc_first = (e0 == plan.first && plan.accumulate_first) ? 1 : 0;
+        dim3 grid((unsigned)ceil_div(out_feat, 64), (unsigned)tab.n);
+        ProfileScope prof(kProfBiasGrad, (double)(tab.seg[tab.n] - tab.seg[0]) * out_feat * dtype_bytes(dtype), stream);
+        switch (dtype) {
+            case FMOE_BF16: bias_grad_kernel<__bf16, float><<<grid, kThreads, 0, stream>>>((const __bf16 *)gy, (__bf16 *)gb, out_feat, tab, acc_first); break;
+            case FMOE_F16: bias_grad_kernel<_Float16, float><<<grid, kThreads, 0, stream>>>((const _Float16 *)gy, (_Float16 *)gb, out_feat, tab, acc_first); break;
+            case FMOE_F32: bias_grad_kernel<float, float><<<grid, kThreads, 0, stream>>>((const float *)gy, (float *)gb, out_feat, tab, acc_first); break;
+            case FMOE_F64: bias_grad_kernel<double, double><<<grid, kThreads, 0, stream>>>((const double *)gy, (double *)gb, out_feat, tab, acc_first); break;
+            default: return fail(FMOE_EINVAL, "bias_grad: unknown dtype %d", dtype);
+        }
+        FMOE_LAUNCH_CHECK();
+    }
+    return FMOE_OK;
+}
+
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" int fmoe_linear_forward(const void *x, const void *w, const void *bias, void *y,
+                                   const int64_t *expert_count_host, int64_t n_expert, int64_t in_feat,
+                                   int64_t out_feat, int dtype, void *stream) {
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_forward: unknown dtype %d", dtype);
+    int64_t total;
+    if (int rc = check_counts("fmoe_linear_forward", expert_count_host, n_expert, 0, 0, &total)) return rc;
+    LinearForwardArgs a{x, w, bias, y, nullptr, in_feat, out_feat, dtype, kEpiStore, FMOE_ACT_NONE};
+    return grouped_linear_forward(a, expert_count_host, n_expert, 0, total, (hipStream_t)stream);
+}
+
+extern "C" int fmoe_linear_backward(const void *grad_y, const void *x, const void *w, void *grad_x, void *grad_w,
+                                    void *grad_b, const int64_t *expert_count_host, int64_t n_expert,
+                                    int64_t in_feat, int64_t out_feat, int dtype, void *stream) {
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_backward: unknown dtype %d", dtype);
+    int64_t total;
+    if (int rc = check_counts("fmoe_linear_backward", expert_count_host, n_expert, 0, 0, &total)) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    if (grad_x) {
+        LinearDgradArgs d{grad_y, w, grad_x, nullptr, in_feat, out_feat, dtype, kEpiStore, FMOE_ACT_NONE};
+        if (int rc = grouped_linear_dgrad(d, expert_count_host, n_expert, 0, total, st)) return rc;
+    }
+    if (grad_w) {
+        LinearWgradArgs g{grad_y, x, grad_w, in_feat, out_feat, dtype};
+        if (int rc = grouped_linear_wgrad(g, expert_count_host, n_expert, 0, total, true, st)) return rc;
+    }
+    if (grad_b)
+        if (int rc = grouped_bias_grad(grad_y, grad_b, out_feat, dtype, expert_count_host, n_expert, 0, total, true, st))
+            return rc;
+    return FMOE_OK;
+}

@@ -1,0 +1,72 @@
+// Grouped GEMM over ragged expert segments (gfx950): host-side interface shared
+// by the per-expert linear entry points and the fused MLP pipeline.
+#pragma once
+#include "common.hpp"
+
+namespace fmoe {
+
+// What the epilogue does with the fp32 accumulator tile.
+enum Epilogue {
+    kEpiStore = 0,    // C = acc (+ bias[col])
+    kEpiBiasAct = 1,  // pre = acc + bias[col]; aux = pre (if aux); C = act(pre)
+    kEpiDAct = 2,     // C = acc * act'(aux)          (aux = saved pre-activation)
+};
+
+constexpr int kMaxGroupExperts = 256;  // experts per launch (table lives in kernel arguments)
+
+// Row segments of the experts covered by one launch.  seg[i] .. seg[i+1] are the
+// rows of expert first_expert + i; for a chunk of the fused pipeline the rows
+// are already clipped to the chunk.
+struct SegmentTable {
+    int32_t n;                            // experts in this launch
+    int32_t first_expert;                 // global index of seg[0]'s expert
+    int32_t seg[kMaxGroupExperts + 1];    // row offsets
+    int32_t tile[kMaxGroupExperts + 1];   // prefix of row tiles (ragged-M launches)
+};
+
+struct LinearForwardArgs {
+    const void *x;      // [rows, in]
+    const void *w;      // [E, out, in]
+    const void *bias;   // [E, out] or null
+    void *y;            // [rows, out]
+    void *aux;          // [rows, out] pre-activation copy (kEpiBiasAct) or null
+    int64_t in_feat, out_feat;
+    int dtype, epilogue, activation;
+};
+
+struct LinearDgradArgs {
+    const void *gy;     // [rows, out]
+    const void *w;      // [E, out, in]
+    void *gx;           // [rows, in]
+    const void *aux;    // [rows, in] pre-activation (kEpiDAct) or null
+    int64_t in_feat, out_feat;
+    int dtype, epilogue, activation;
+};
+
+struct LinearWgradArgs {
+    const void *gy;     // [rows, out]
+    const void *x;      // [rows, in]
+    void *gw;           // [E, out, in]
+    int64_t in_feat, out_feat;
+    int dtype;
+};
+
+// counts[e] rows for experts [0, n_expert), restricted to rows [row_lo, row_hi)
+// of the expert-sorted order.  Launches on `stream`; for more than
+// kMaxGroupExperts experts the work is split into several launches.
+int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts_host, int64_t n_expert,
+                           int64_t row_lo, int64_t row_hi, hipStream_t stream);
+int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts_host, int64_t n_expert,
+                         int64_t row_lo, int64_t row_hi, hipStream_t stream);
+// Weight gradient over the rows [row_lo, row_hi).  An expert is written by the
+// chunk that holds any of its rows; an expert without rows is zero-filled by
+// the chunk that contains its (empty) position, the last chunk taking the
+// position row_hi.  An expert whose rows began before row_lo adds to what the
+// earlier chunk left (cuda/fused_compute.cuh:123, beta_weight).
+int grouped_linear_wgrad(const LinearWgradArgs &a, const int64_t *counts_host, int64_t n_expert,
+                         int64_t row_lo, int64_t row_hi, bool last_chunk, hipStream_t stream);
+// grad_b[e, c] = column sums of gy over the rows of expert e; same chunk rules.
+int grouped_bias_grad(const void *gy, void *gb, int64_t out_feat, int dtype, const int64_t *counts_host,
+                      int64_t n_expert, int64_t row_lo, int64_t row_hi, bool last_chunk, hipStream_t stream);
+
+}  // namespace fmoe

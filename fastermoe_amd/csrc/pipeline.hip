@@ -1,0 +1,231 @@
+// Fused expert-MLP pipeline for one worker (gfx950).
+//
+// The expert-sorted rows are cut into `n_chunks` contiguous chunks.  Three HIP
+// streams owned by the library run, for chunk c,
+//     permute-in  : gather token rows into the sorted buffer
+//     compute     : grouped GEMM 1 (+bias, activation), grouped GEMM 2 (+bias)
+//     permute-out : write expert outputs back to slot order
+// so that chunk c+1's permute-in and chunk c-1's permute-out overlap chunk c's
+// GEMMs.  Chunks are chained by events (in_ready[c], out_ready[c]); the
+// caller's stream forks into the three streams at entry and joins them at
+// exit, so the call behaves like one asynchronous operation on that stream.
+// Backward mirrors this: gather grad rows, dgrad/wgrad of both linears with the
+// activation derivative folded into the first dgrad's epilogue, and a final
+// per-token reduction of the k expert-row gradients.
+//
+// All streams use the default priority.  Events are created once per device and
+// reused; a call therefore must not overlap another call of this library's fused
+// entry points on the same device from a different host thread.
+#include "grouped_gemm.hpp"
+#include "permute.hpp"
+
+#include <mutex>
+#include <vector>
+
+namespace fmoe {
+namespace {
+
+constexpr int kMaxChunks = 32;
+
+struct DeviceLanes {
+    bool ready = false;
+    hipStream_t in = nullptr, compute = nullptr, out = nullptr;
+    hipEvent_t fork = nullptr, join_in = nullptr, join_compute = nullptr, join_out = nullptr;
+    hipEvent_t in_ready[kMaxChunks] = {};
+    hipEvent_t out_ready[kMaxChunks] = {};
+};
+
+std::mutex g_lanes_mutex;
+DeviceLanes g_lanes[16];
+
+int get_lanes(DeviceLanes **out) {
+    int dev = 0;
+    FMOE_HIP_CHECK(hipGetDevice(&dev));
+    FMOE_REQUIRE(dev >= 0 && dev < 16, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_lanes_mutex);
+    DeviceLanes &l = g_lanes[dev];
+    if (!l.ready) {
+        FMOE_HIP_CHECK(hipStreamCreateWithFlags(&l.in, hipStreamNonBlocking));
+        FMOE_HIP_CHECK(hipStreamCreateWithFlags(&l.compute, hipStreamNonBlocking));
+        FMOE_HIP_CHECK(hipStreamCreateWithFlags(&l.out, hipStreamNonBlocking));
+        hipEvent_t *single[] = {&l.fork, &l.join_in, &l.join_compute, &l.join_out};
+        for (hipEvent_t *e : single) FMOE_HIP_CHECK(hipEventCreateWithFlags(e, hipEventDisableTiming));
+        for (int c = 0; c < kMaxChunks; ++c) {
+            FMOE_HIP_CHECK(hipEventCreateWithFlags(&l.in_ready[c], hipEventDisableTiming));
+            FMOE_HIP_CHECK(hipEventCreateWithFlags(&l.out_ready[c], hipEventDisableTiming));
+        }
+        l.ready = true;
+    }
+    *out = &l;
+    return FMOE_OK;
+}
+
+int fork_lanes(DeviceLanes *l, hipStream_t caller) {
+    FMOE_HIP_CHECK(hipEventRecord(l->fork, caller));
+    FMOE_HIP_CHECK(hipStreamWaitEvent(l->in, l->fork, 0));
+    FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->fork, 0));
+    FMOE_HIP_CHECK(hipStreamWaitEvent(l->out, l->fork, 0));
+    return FMOE_OK;
+}
+
+int join_lanes(DeviceLanes *l, hipStream_t caller) {
+    FMOE_HIP_CHECK(hipEventRecord(l->join_in, l->in));
+    FMOE_HIP_CHECK(hipEventRecord(l->join_compute, l->compute));
+    FMOE_HIP_CHECK(hipEventRecord(l->join_out, l->out));
+    FMOE_HIP_CHECK(hipStreamWaitEvent(caller, l->join_in, 0));
+    FMOE_HIP_CHECK(hipStreamWaitEvent(caller, l->join_compute, 0));
+    FMOE_HIP_CHECK(hipStreamWaitEvent(caller, l->join_out, 0));
+    return FMOE_OK;
+}
+
+int check_common(const char *who, const fmoe_mlp_params *p, const int64_t *counts, int64_t n_tokens,
+                 int64_t top_k, int64_t n_rows, int n_chunks) {
+    FMOE_REQUIRE(p != nullptr, "%s: params is NULL", who);
+    FMOE_REQUIRE(p->dtype == FMOE_F32 || p->dtype == FMOE_BF16 || p->dtype == FMOE_F16,
+                 "%s: dtype %d not supported by the fused path (f32, bf16, f16)", who, p->dtype);
+    FMOE_REQUIRE(p->activation >= FMOE_ACT_NONE && p->activation <= FMOE_ACT_GELU, "%s: activation %d", who,
+                 p->activation);
+    FMOE_REQUIRE(p->n_expert >= 1 && p->d_model >= 1 && p->d_hidden >= 1, "%s: bad sizes", who);
+    FMOE_REQUIRE(p->w1 && p->w2, "%s: NULL weights", who);
+    FMOE_REQUIRE(n_tokens >= 0 && top_k >= 1 && n_rows >= 0 && n_rows <= n_tokens * top_k,
+                 "%s: n_tokens=%lld top_k=%lld n_rows=%lld", who, (long long)n_tokens, (long long)top_k,
+                 (long long)n_rows);
+    FMOE_REQUIRE(n_chunks >= 1 && n_chunks <= kMaxChunks, "%s: n_chunks=%d (1..%d)", who, n_chunks, kMaxChunks);
+    FMOE_REQUIRE(counts != nullptr, "%s: expert_count_host is NULL", who);
+    int64_t s = 0;
+    for (int64_t e = 0; e < p->n_expert; ++e) {
+        FMOE_REQUIRE(counts[e] >= 0, "%s: negative expert count", who);
+        s += counts[e];
+    }
+    FMOE_REQUIRE(s == n_rows, "%s: expert counts sum to %lld, n_rows is %lld", who, (long long)s,
+                 (long long)n_rows);
+    return FMOE_OK;
+}
+
+inline const char *at(const void *base, int64_t row, int64_t row_elems, int dtype) {
+    return static_cast<const char *>(base) + row * row_elems * dtype_bytes(dtype);
+}
+inline char *at(void *base, int64_t row, int64_t row_elems, int dtype) {
+    return static_cast<char *>(base) + row * row_elems * dtype_bytes(dtype);
+}
+
+}  // namespace
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp, const int64_t *pos,
+                                      const int64_t *slot_to_row, const int64_t *expert_count_host,
+                                      int64_t n_tokens, int64_t top_k, int64_t n_rows, void *buf_in,
+                                      void *buf_pre, void *buf_mid, void *buf_out, void *out, int n_chunks,
+                                      void *stream) {
+    if (int rc = check_common("fmoe_fused_mlp_forward", p, expert_count_host, n_tokens, top_k, n_rows, n_chunks))
+        return rc;
+    const int64_t n_slots = n_tokens * top_k;
+    if (n_slots == 0) return FMOE_OK;
+    FMOE_REQUIRE(out && slot_to_row, "fmoe_fused_mlp_forward: NULL out / slot_to_row");
+    FMOE_REQUIRE(n_rows == 0 || (inp && pos && buf_in && buf_mid && buf_out),
+                 "fmoe_fused_mlp_forward: NULL buffer");
+    const int dt = p->dtype;
+    const int64_t d = p->d_model, h = p->d_hidden, E = p->n_expert;
+    hipStream_t caller = (hipStream_t)stream;
+    DeviceLanes *l;
+    if (int rc = get_lanes(&l)) return rc;
+    if (int rc = fork_lanes(l, caller)) return rc;
+
+    // dropped slots become zero rows; independent of everything else
+    if (n_rows < n_slots)
+        if (int rc = permute_zero_unmapped(slot_to_row, out, n_slots, d, dt, l->out)) return rc;
+
+    for (int c = 0; c < n_chunks; ++c) {
+        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        if (hi == lo) continue;
+        // permute-in: buf_in[r] = inp[pos[r] / top_k]
+        if (int rc = permute_gather_rows(inp, pos + lo, top_k, at(buf_in, lo, d, dt), hi - lo, n_tokens, d, dt, l->in))
+            return rc;
+        FMOE_HIP_CHECK(hipEventRecord(l->in_ready[c], l->in));
+    }
+    for (int c = 0; c < n_chunks; ++c) {
+        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        if (hi == lo) continue;
+        FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
+        LinearForwardArgs f1{buf_in, p->w1, p->b1, buf_mid, buf_pre, d, h, dt, kEpiBiasAct, p->activation};
+        if (int rc = grouped_linear_forward(f1, expert_count_host, E, lo, hi, l->compute)) return rc;
+        LinearForwardArgs f2{buf_mid, p->w2, p->b2, buf_out, nullptr, h, d, dt, kEpiStore, FMOE_ACT_NONE};
+        if (int rc = grouped_linear_forward(f2, expert_count_host, E, lo, hi, l->compute)) return rc;
+        FMOE_HIP_CHECK(hipEventRecord(l->out_ready[c], l->compute));
+    }
+    for (int c = 0; c < n_chunks; ++c) {
+        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        if (hi == lo) continue;
+        FMOE_HIP_CHECK(hipStreamWaitEvent(l->out, l->out_ready[c], 0));
+        // permute-out: out[pos[r]] = buf_out[r]
+        if (int rc = permute_scatter_rows(at(buf_out, lo, d, dt), pos + lo, out, hi - lo, n_slots, d, dt, l->out))
+            return rc;
+    }
+    return join_lanes(l, caller);
+}
+
+extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *grad_out, const int64_t *pos,
+                                       const int64_t *slot_to_row, const int64_t *expert_count_host,
+                                       int64_t n_tokens, int64_t top_k, int64_t n_rows, const void *buf_in,
+                                       const void *buf_pre, const void *buf_mid, void *g_out, void *g_mid,
+                                       void *g_in, void *grad_inp, void *grad_w1, void *grad_b1, void *grad_w2,
+                                       void *grad_b2, int n_chunks, void *stream) {
+    if (int rc = check_common("fmoe_fused_mlp_backward", p, expert_count_host, n_tokens, top_k, n_rows, n_chunks))
+        return rc;
+    FMOE_REQUIRE(grad_w1 && grad_w2, "fmoe_fused_mlp_backward: NULL weight gradient");
+    FMOE_REQUIRE(n_tokens == 0 || (grad_inp && slot_to_row), "fmoe_fused_mlp_backward: NULL grad_inp / slot_to_row");
+    FMOE_REQUIRE(n_rows == 0 || (grad_out && pos && buf_in && buf_mid && g_out && g_mid && g_in),
+                 "fmoe_fused_mlp_backward: NULL buffer");
+    FMOE_REQUIRE(p->activation == FMOE_ACT_NONE || n_rows == 0 || buf_pre,
+                 "fmoe_fused_mlp_backward: pre-activation buffer is NULL");
+    const int dt = p->dtype;
+    const int64_t d = p->d_model, h = p->d_hidden, E = p->n_expert;
+    const int64_t n_slots = n_tokens * top_k;
+    hipStream_t caller = (hipStream_t)stream;
+    DeviceLanes *l;
+    if (int rc = get_lanes(&l)) return rc;
+    if (int rc = fork_lanes(l, caller)) return rc;
+
+    for (int c = 0; c < n_chunks; ++c) {
+        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        if (hi == lo) continue;
+        // permute-in: g_out[r] = grad_out[pos[r]]
+        if (int rc = permute_gather_rows(grad_out, pos + lo, 1, at(g_out, lo, d, dt), hi - lo, n_slots, d, dt, l->in))
+            return rc;
+        FMOE_HIP_CHECK(hipEventRecord(l->in_ready[c], l->in));
+    }
+    // The last chunk (even when it is empty) also zero-fills the experts without rows.
+    int last = n_chunks - 1;
+    for (int c = 0; c < n_chunks; ++c) {
+        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        const bool is_last = c == last;
+        if (hi == lo && !is_last) continue;
+        if (hi > lo) FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
+        // second linear: g_mid = (g_out . W2) * act'(pre);  gW2 (+)= g_out^T . mid;  gb2 (+)= colsum(g_out)
+        const bool has_act = p->activation != FMOE_ACT_NONE;
+        LinearDgradArgs d2{g_out, p->w2, g_mid, has_act ? buf_pre : nullptr, h, d, dt,
+                           has_act ? kEpiDAct : kEpiStore, p->activation};
+        if (int rc = grouped_linear_dgrad(d2, expert_count_host, E, lo, hi, l->compute)) return rc;
+        LinearWgradArgs w2{g_out, buf_mid, grad_w2, h, d, dt};
+        if (int rc = grouped_linear_wgrad(w2, expert_count_host, E, lo, hi, is_last, l->compute)) return rc;
+        if (grad_b2)
+            if (int rc = grouped_bias_grad(g_out, grad_b2, d, dt, expert_count_host, E, lo, hi, is_last, l->compute))
+                return rc;
+        // first linear: g_in = g_mid . W1;  gW1 (+)= g_mid^T . buf_in;  gb1 (+)= colsum(g_mid)
+        LinearDgradArgs d1{g_mid, p->w1, g_in, nullptr, d, h, dt, kEpiStore, FMOE_ACT_NONE};
+        if (int rc = grouped_linear_dgrad(d1, expert_count_host, E, lo, hi, l->compute)) return rc;
+        LinearWgradArgs w1{g_mid, buf_in, grad_w1, d, h, dt};
+        if (int rc = grouped_linear_wgrad(w1, expert_count_host, E, lo, hi, is_last, l->compute)) return rc;
+        if (grad_b1)
+            if (int rc = grouped_bias_grad(g_mid, grad_b1, h, dt, expert_count_host, E, lo, hi, is_last, l->compute))
+                return rc;
+    }
+    if (int rc = join_lanes(l, caller)) return rc;
+    // grad_inp[t] = sum of the token's k expert-row gradients (rows of different
+    // chunks, so this runs once, after all of them)
+    if (n_tokens > 0)
+        if (int rc = fmoe_reduce_slots(g_in, slot_to_row, grad_inp, n_tokens, top_k, n_rows, d, dt, caller)) return rc;
+    return FMOE_OK;
+}

@@ -1,0 +1,390 @@
+// Routing bookkeeping and capacity balancing for gfx950.
+//
+// Every entry point that has to order slots ("which slots of expert e come
+// first") is built on one primitive: the RANK of a slot among the slots of the
+// same expert with a lower flat index.  The rank is computed without atomics on
+// shared counters, so results do not depend on scheduling:
+//
+//   1. hist   : each 256-thread workgroup owns kSlotsPerBlock consecutive slots
+//               and writes its per-expert histogram (LDS-staged) to scratch;
+//   2. scan   : per expert, an exclusive prefix over the workgroups (and, for
+//               fmoe_route, the cumsum over experts);
+//   3. apply  : each wave walks its 512 slots in order; inside a 64-slot step
+//               the rank comes from a ballot-built match mask and a popcount of
+//               the lower lanes, across steps from a wave-private LDS counter.
+//
+// The index arrays are a few hundred KB at most, so these kernels are bound by
+// launch and memory latency, not by HBM bandwidth; the design keeps them to
+// three short launches with coalesced 8-byte loads.
+#include "common.hpp"
+
+namespace fmoe {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kStepsPerWave = 8;
+constexpr int kSlotsPerWave = kWave * kStepsPerWave;          // 512
+constexpr int kSlotsPerBlock = kSlotsPerWave * kWavesPerBlock; // 2048
+constexpr int64_t kMaxExpert = 8192;  // 4 wave-private int32 tables in 160 KB LDS
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+__device__ __forceinline__ uint64_t lanes_below() {
+    return (1ull << lane_id()) - 1ull;
+}
+
+// Mask of the lanes of this wave that hold the same key; lanes with
+// valid == false get 0.  nbits = number of significant key bits.
+__device__ __forceinline__ uint64_t match_mask(int key, bool valid, int nbits) {
+    uint64_t peers = __ballot(valid);
+    for (int b = 0; b < nbits; ++b) {
+        const bool bit = (key >> b) & 1;
+        const uint64_t vote = __ballot(valid && bit);
+        peers &= bit ? vote : ~vote;
+    }
+    return valid ? peers : 0ull;
+}
+
+// ---------------------------------------------------------------- count ----
+
+// LDS histogram per workgroup, one global integer add per non-empty bin.
+__global__ __launch_bounds__(kBlock) void expert_count_kernel(
+    const int64_t *__restrict__ gate, int32_t *__restrict__ count,
+    int64_t n_slots, int n_expert) {
+    extern __shared__ int32_t bins[];
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) bins[e] = 0;
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n_slots; i += stride) {
+        const int64_t g = gate[i];
+        if (g >= 0 && g < n_expert) atomicAdd(&bins[(int)g], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) {
+        const int32_t c = bins[e];
+        if (c) atomicAdd(&count[e], c);
+    }
+}
+
+// ----------------------------------------------------------------- hist ----
+
+// block_hist[b][e] = #slots of expert e in workgroup b's slot range.
+__global__ __launch_bounds__(kBlock) void block_hist_kernel(
+    const int64_t *__restrict__ gate, int32_t *__restrict__ block_hist,
+    int64_t n_slots, int n_expert) {
+    extern __shared__ int32_t bins[];
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) bins[e] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kSlotsPerBlock;
+#pragma unroll
+    for (int s = 0; s < kSlotsPerBlock / kBlock; ++s) {
+        const int64_t i = base + s * kBlock + threadIdx.x;
+        if (i < n_slots) {
+            const int64_t g = gate[i];
+            if (g >= 0 && g < n_expert) atomicAdd(&bins[(int)g], 1);
+        }
+    }
+    __syncthreads();
+    int32_t *dst = block_hist + (int64_t)blockIdx.x * n_expert;
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) dst[e] = bins[e];
+}
+
+// ----------------------------------------------------------------- scan ----
+
+enum ScanMode { kScanAssign = 0, kScanPrune = 1 };
+
+// One thread per expert: block_hist[.][e] -> exclusive prefix over workgroups
+// (in place).  limit[e] is the caller's per-expert int32 array (cum_count for
+// assign_pos, remaining capacity for prune); its old value is parked in
+// limit_old[e] for the apply kernel and the array is updated the way the
+// reference kernel leaves it (every slot subtracts one).
+__global__ __launch_bounds__(kBlock) void block_scan_kernel(
+    int32_t *__restrict__ block_hist, int n_blocks, int n_expert,
+    int32_t *__restrict__ limit, int32_t *__restrict__ limit_old) {
+    const int e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= n_expert) return;
+    int32_t run = 0;
+    for (int b = 0; b < n_blocks; ++b) {
+        int32_t *cell = block_hist + (int64_t)b * n_expert + e;
+        const int32_t c = *cell;
+        *cell = run;
+        run += c;
+    }
+    const int32_t old = limit[e];
+    limit_old[e] = old;
+    limit[e] = old - run;
+}
+
+// fmoe_route: a single 1024-thread workgroup does the per-expert prefix over
+// workgroups and then the inclusive cumsum over experts.
+constexpr int kRouteScanBlock = 1024;
+__global__ __launch_bounds__(kRouteScanBlock) void route_scan_kernel(
+    int32_t *__restrict__ block_hist, int n_blocks, int n_expert,
+    int64_t *__restrict__ expert_count, int32_t *__restrict__ cum_incl) {
+    __shared__ int32_t wave_sum[kRouteScanBlock / kWave];
+    __shared__ int32_t carry_s;
+    if (threadIdx.x == 0) carry_s = 0;
+    __syncthreads();
+    for (int e0 = 0; e0 < n_expert; e0 += kRouteScanBlock) {
+        const int e = e0 + threadIdx.x;
+        int32_t run = 0;
+        if (e < n_expert) {
+            for (int b = 0; b < n_blocks; ++b) {
+                int32_t *cell = block_hist + (int64_t)b * n_expert + e;
+                const int32_t c = *cell;
+                *cell = run;
+                run += c;
+            }
+            expert_count[e] = run;
+        }
+        // inclusive scan of `run` over the workgroup
+        int32_t v = run;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int32_t up = __shfl_up(v, off, kWave);
+            if (lane_id() >= off) v += up;
+        }
+        const int wave = threadIdx.x / kWave;
+        if (lane_id() == kWave - 1) wave_sum[wave] = v;
+        __syncthreads();
+        int32_t before = carry_s;
+        for (int w = 0; w < wave; ++w) before += wave_sum[w];
+        if (e < n_expert) cum_incl[e] = v + before;
+        __syncthreads();
+        if (threadIdx.x == kRouteScanBlock - 1) carry_s = v + before;
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------- apply ----
+
+enum ApplyMode { kApplyAssign = 0, kApplyPrune = 1 };
+
+// Recomputes the per-wave histograms of this workgroup's slots, turns them into
+// per-wave starting ranks (block prefix from the scan + waves before this one)
+// and walks the slots in order.
+//   assign: pos[limit_old[e] - 1 - rank] = slot   (+ slot_to_row[slot] = that)
+//   prune : out[slot] = rank < limit_old[e] ? e : -1
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void rank_apply_kernel(
+    const int64_t *__restrict__ gate, const int32_t *__restrict__ block_base,
+    const int32_t *__restrict__ limit_old, int64_t *__restrict__ out,
+    int64_t *__restrict__ slot_to_row, int64_t n_slots, int64_t n_out, int n_expert, int nbits) {
+    extern __shared__ int32_t lds[];  // [kWavesPerBlock][n_expert]
+    const int wave = threadIdx.x / kWave;
+    int32_t *mine = lds + wave * n_expert;
+    for (int e = threadIdx.x; e < kWavesPerBlock * n_expert; e += kBlock) lds[e] = 0;
+    __syncthreads();
+
+    const int64_t wave_base = (int64_t)blockIdx.x * kSlotsPerBlock + (int64_t)wave * kSlotsPerWave;
+    int keys[kStepsPerWave];
+#pragma unroll
+    for (int s = 0; s < kStepsPerWave; ++s) {
+        const int64_t i = wave_base + s * kWave + lane_id();
+        int64_t g = -1;
+        if (i < n_slots) g = gate[i];
+        keys[s] = (g >= 0 && g < n_expert) ? (int)g : -1;
+        if (keys[s] >= 0) atomicAdd(&mine[keys[s]], 1);
+    }
+    __syncthreads();
+    // per-wave histogram -> starting rank of this wave for every expert
+    const int32_t *bb = block_base + (int64_t)blockIdx.x * n_expert;
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) {
+        int32_t run = bb[e];
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) {
+            const int32_t c = lds[w * n_expert + e];
+            lds[w * n_expert + e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int s = 0; s < kStepsPerWave; ++s) {
+        const int64_t i = wave_base + s * kWave + lane_id();
+        const int key = keys[s];
+        const bool valid = key >= 0;
+        const uint64_t peers = match_mask(key, valid, nbits);
+        int32_t rank = 0;
+        if (valid) rank = mine[key] + __popcll(peers & lanes_below());
+        __syncthreads();  // every lane has read its counter before leaders bump it
+        if (valid && (peers & lanes_below()) == 0) mine[key] += __popcll(peers);
+        __syncthreads();
+        if (MODE == kApplyAssign) {
+            if (valid) {
+                const int64_t row = (int64_t)limit_old[key] - 1 - rank;
+                if (row >= 0 && row < n_out) out[row] = i;  // a short pos buffer is never overrun
+                if (slot_to_row) slot_to_row[i] = row;
+            } else if (slot_to_row && i < n_slots) {
+                slot_to_row[i] = -1;
+            }
+        } else {
+            if (i < n_slots) out[i] = (valid && rank < limit_old[key]) ? (int64_t)key : -1;
+        }
+    }
+}
+
+// ------------------------------------------------------------- capacity ----
+
+// One thread per expert, workers in ascending order (the order that fixes who
+// gets the remaining capacity).
+__global__ __launch_bounds__(kBlock) void limit_by_capacity_kernel(
+    const int64_t *__restrict__ ec, int32_t *__restrict__ cap, int64_t *__restrict__ eca,
+    int64_t n_expert, int64_t n_worker) {
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= n_expert) return;
+    int32_t left = cap[e];
+    for (int64_t w = 0; w < n_worker; ++w) {
+        const int32_t proposal = (int32_t)ec[w * n_expert + e];
+        int64_t grant;
+        if (left >= proposal) grant = proposal;
+        else if (left >= 0) grant = left;
+        else grant = 0;
+        eca[w * n_expert + e] = grant;
+        left -= proposal;
+    }
+    cap[e] = left;
+}
+
+int ilog2_ceil(int64_t n) {
+    int b = 0;
+    while ((1ll << b) < n) ++b;
+    return b < 1 ? 1 : b;
+}
+
+struct RouteScratch {
+    int32_t *block_hist;  // [n_blocks][n_expert]
+    int32_t *limit_old;   // [n_expert]
+    int32_t *cum;         // [n_expert]  (fmoe_route only)
+    int n_blocks;
+};
+
+int64_t scratch_bytes(int64_t n_slots, int64_t n_expert) {
+    const int64_t nb = ceil_div(n_slots > 0 ? n_slots : 1, kSlotsPerBlock);
+    return (nb * n_expert + 2 * n_expert) * (int64_t)sizeof(int32_t) + 64;
+}
+
+int carve(void *workspace, int64_t workspace_bytes, int64_t n_slots, int64_t n_expert, RouteScratch *s) {
+    const int64_t need = scratch_bytes(n_slots, n_expert);
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(FMOE_EWORKSPACE, "routing workspace: need %lld bytes, got %lld",
+                    (long long)need, (long long)workspace_bytes);
+    FMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, "routing workspace must be 4-byte aligned");
+    const int64_t nb = ceil_div(n_slots > 0 ? n_slots : 1, kSlotsPerBlock);
+    s->block_hist = static_cast<int32_t *>(workspace);
+    s->limit_old = s->block_hist + nb * n_expert;
+    s->cum = s->limit_old + n_expert;
+    s->n_blocks = (int)nb;
+    return FMOE_OK;
+}
+
+int check_sizes(int64_t n_slots, int64_t n_expert) {
+    FMOE_REQUIRE(n_slots >= 0, "n_slots must be >= 0 (got %lld)", (long long)n_slots);
+    FMOE_REQUIRE(n_expert >= 1, "n_expert must be >= 1 (got %lld)", (long long)n_expert);
+    if (n_expert > kMaxExpert)
+        return fail(FMOE_ELIMIT, "n_expert %lld exceeds the supported maximum %lld",
+                    (long long)n_expert, (long long)kMaxExpert);
+    if (n_slots > (int64_t)INT32_MAX)
+        return fail(FMOE_ELIMIT, "n_slots %lld exceeds int32 range", (long long)n_slots);
+    return FMOE_OK;
+}
+
+}  // namespace
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" int fmoe_expert_count(const int64_t *gate_idx, int32_t *expert_count, int64_t n_slots,
+                                 int64_t n_expert, void *stream) {
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    if (n_slots == 0) return FMOE_OK;
+    FMOE_REQUIRE(gate_idx && expert_count, "fmoe_expert_count: NULL pointer");
+    const int64_t blocks = ceil_div(n_slots, (int64_t)kBlock * 8);
+    const int grid = (int)(blocks < 1024 ? blocks : 1024);
+    expert_count_kernel<<<grid, kBlock, n_expert * sizeof(int32_t), (hipStream_t)stream>>>(
+        gate_idx, expert_count, n_slots, (int)n_expert);
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+extern "C" int64_t fmoe_routing_workspace_bytes(int64_t n_slots, int64_t n_expert) {
+    if (n_slots < 0 || n_expert < 1) return 0;
+    return scratch_bytes(n_slots, n_expert);
+}
+
+extern "C" int fmoe_assign_pos(int32_t *cum_count, const int64_t *gate, int64_t *pos, int64_t n_pos,
+                               int64_t n_slots, int64_t n_expert, void *workspace, int64_t workspace_bytes,
+                               void *stream) {
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    if (n_slots == 0) return FMOE_OK;
+    FMOE_REQUIRE(cum_count && gate && n_pos >= 0 && (pos || n_pos == 0), "fmoe_assign_pos: NULL pointer");
+    RouteScratch s;
+    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const int E = (int)n_expert;
+    block_hist_kernel<<<s.n_blocks, kBlock, E * sizeof(int32_t), st>>>(gate, s.block_hist, n_slots, E);
+    FMOE_LAUNCH_CHECK();
+    block_scan_kernel<<<(int)ceil_div(E, kBlock), kBlock, 0, st>>>(s.block_hist, s.n_blocks, E, cum_count, s.limit_old);
+    FMOE_LAUNCH_CHECK();
+    rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
+        gate, s.block_hist, s.limit_old, pos, nullptr, n_slots, n_pos, E, ilog2_ceil(n_expert));
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_route(const int64_t *gate, int64_t n_slots, int64_t n_expert, int64_t *expert_count,
+                          int64_t *pos, int64_t *slot_to_row, void *workspace, int64_t workspace_bytes,
+                          void *stream) {
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    FMOE_REQUIRE(expert_count, "fmoe_route: NULL expert_count");
+    hipStream_t st = (hipStream_t)stream;
+    if (n_slots == 0) {
+        FMOE_HIP_CHECK(hipMemsetAsync(expert_count, 0, n_expert * sizeof(int64_t), st));
+        return FMOE_OK;
+    }
+    FMOE_REQUIRE(gate && pos, "fmoe_route: NULL pointer");
+    RouteScratch s;
+    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+    const int E = (int)n_expert;
+    block_hist_kernel<<<s.n_blocks, kBlock, E * sizeof(int32_t), st>>>(gate, s.block_hist, n_slots, E);
+    FMOE_LAUNCH_CHECK();
+    route_scan_kernel<<<1, kRouteScanBlock, 0, st>>>(s.block_hist, s.n_blocks, E, expert_count, s.cum);
+    FMOE_LAUNCH_CHECK();
+    rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
+        gate, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert));
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_limit_by_capacity(const int64_t *ec, int32_t *cap, int64_t *eca, int64_t n_expert,
+                                      int64_t n_worker, void *stream) {
+    FMOE_REQUIRE(n_expert >= 1 && n_worker >= 1, "fmoe_limit_by_capacity: n_expert=%lld n_worker=%lld",
+                 (long long)n_expert, (long long)n_worker);
+    FMOE_REQUIRE(ec && cap && eca, "fmoe_limit_by_capacity: NULL pointer");
+    limit_by_capacity_kernel<<<(int)ceil_div(n_expert, kBlock), kBlock, 0, (hipStream_t)stream>>>(
+        ec, cap, eca, n_expert, n_worker);
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_prune_gate_by_capacity(const int64_t *gate_idx, int64_t *new_gate_idx, int32_t *ec,
+                                           int64_t n_slots, int64_t n_expert, void *workspace,
+                                           int64_t workspace_bytes, void *stream) {
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    if (n_slots == 0) return FMOE_OK;
+    FMOE_REQUIRE(gate_idx && new_gate_idx && ec, "fmoe_prune_gate_by_capacity: NULL pointer");
+    RouteScratch s;
+    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const int E = (int)n_expert;
+    block_hist_kernel<<<s.n_blocks, kBlock, E * sizeof(int32_t), st>>>(gate_idx, s.block_hist, n_slots, E);
+    FMOE_LAUNCH_CHECK();
+    block_scan_kernel<<<(int)ceil_div(E, kBlock), kBlock, 0, st>>>(s.block_hist, s.n_blocks, E, ec, s.limit_old);
+    FMOE_LAUNCH_CHECK();
+    rank_apply_kernel<kApplyPrune><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
+        gate_idx, s.block_hist, s.limit_old, new_gate_idx, nullptr, n_slots, n_slots, E, ilog2_ceil(n_expert));
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}

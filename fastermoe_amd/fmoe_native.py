@@ -1,0 +1,384 @@
+"""Operator module with the interface of the reference's ``fmoe_cuda`` extension
+(cuda/fmoe_cuda.cpp:105-130), backed by ``libfmoe_hip.so``.
+
+Every function validates its tensors (Python exceptions instead of the
+reference's ``exit()``), allocates outputs with torch, and enqueues the HIP
+kernels on torch's current stream through the C ABI.  Nothing here computes on
+the CPU and nothing falls back to torch operators.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import check
+
+_DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16,
+           torch.float64: _lib.F64}
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _dev(name, t, dtype=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a CUDA (HIP) tensor, got device {t.device}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+    return t
+
+
+def _host_counts(name, t, n=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.is_cuda:
+        raise ValueError(f"{name} must be a CPU tensor (it is read on the host)")
+    if t.dtype != torch.int64:
+        raise TypeError(f"{name} must have dtype torch.int64, got {t.dtype}")
+    t = t.contiguous().view(-1)
+    if n is not None and t.numel() != n:
+        raise ValueError(f"{name} has {t.numel()} entries, expected {n}")
+    return t
+
+
+def _float_dtype(name, t):
+    if t.dtype not in _DTYPES:
+        raise TypeError(f"{name}: unsupported dtype {t.dtype}")
+    return _DTYPES[t.dtype]
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+# ---- routing ----------------------------------------------------------------
+
+def expert_count(gate_idx, expert_count):
+    """expert_count[e] += number of entries of gate_idx equal to e (-1 skipped).
+    fmoe_cuda.expert_count, cuda/local_exchange.cu:22-32."""
+    _dev("gate_idx", gate_idx, torch.int64)
+    _dev("expert_count", expert_count, torch.int32)
+    lib = _lib.load()
+    with torch.cuda.device(gate_idx.device):
+        check(lib.fmoe_expert_count(_ptr(gate_idx), _ptr(expert_count), gate_idx.numel(),
+                                    expert_count.numel(), _stream(gate_idx)))
+
+
+def assign_pos(cum_count, gate, pos):
+    """Fills ``pos`` with the slot indices grouped by expert; ``cum_count`` (int32
+    inclusive cumsum) is left as the exclusive cumsum.
+    fmoe_cuda.assign_pos, cuda/local_exchange.cu:5-20."""
+    _dev("cum_count", cum_count, torch.int32)
+    _dev("gate", gate, torch.int64)
+    _dev("pos", pos, torch.int64)
+    lib = _lib.load()
+    n, e = gate.numel(), cum_count.numel()
+    with torch.cuda.device(gate.device):
+        ws = _workspace(lib.fmoe_routing_workspace_bytes(n, e), gate.device)
+        check(lib.fmoe_assign_pos(_ptr(cum_count), _ptr(gate), _ptr(pos), pos.numel(), n, e, _ptr(ws), ws.numel(),
+                                  _stream(gate)))
+
+
+def route(gate, n_expert):
+    """One call for what fmoe/functions.py:19-42 does in several: returns
+    ``(expert_count int64 [E], pos_buf int64 [n_slots], slot_to_row int64 [n_slots])``,
+    all on the device.  Only the first ``expert_count.sum()`` entries of
+    ``pos_buf`` are meaningful."""
+    _dev("gate", gate, torch.int64)
+    lib = _lib.load()
+    n = gate.numel()
+    with torch.cuda.device(gate.device):
+        cnt = torch.empty(n_expert, dtype=torch.int64, device=gate.device)
+        pos = torch.empty(n, dtype=torch.int64, device=gate.device)
+        s2r = torch.empty(n, dtype=torch.int64, device=gate.device)
+        ws = _workspace(lib.fmoe_routing_workspace_bytes(n, n_expert), gate.device)
+        check(lib.fmoe_route(_ptr(gate), n, n_expert, _ptr(cnt), _ptr(pos), _ptr(s2r), _ptr(ws), ws.numel(),
+                             _stream(gate)))
+    return cnt, pos, s2r
+
+
+def limit_by_capacity(expert_count, capacity, n_expert, n_worker):
+    """fmoe_cuda.limit_by_capacity, cuda/balancing.cu:7-20."""
+    _dev("expert_count", expert_count, torch.int64)
+    _dev("capacity", capacity, torch.int32)
+    if expert_count.numel() != n_expert * n_worker:
+        raise ValueError("expert_count must have n_expert * n_worker entries")
+    if capacity.numel() != n_expert:
+        raise ValueError("capacity must have n_expert entries")
+    lib = _lib.load()
+    out = torch.empty_like(expert_count)
+    with torch.cuda.device(expert_count.device):
+        check(lib.fmoe_limit_by_capacity(_ptr(expert_count), _ptr(capacity), _ptr(out), n_expert, n_worker,
+                                         _stream(expert_count)))
+    return out
+
+
+def prune_gate_by_capacity(gate_idx, expert_count, n_expert, n_worker):
+    """fmoe_cuda.prune_gate_by_capacity, cuda/balancing.cu:22-37."""
+    _dev("gate_idx", gate_idx, torch.int64)
+    _dev("expert_count", expert_count, torch.int32)
+    if expert_count.numel() != n_expert * n_worker:
+        raise ValueError("expert_count must have n_expert * n_worker entries")
+    lib = _lib.load()
+    out = torch.empty_like(gate_idx)
+    n, e = gate_idx.numel(), expert_count.numel()
+    with torch.cuda.device(gate_idx.device):
+        ws = _workspace(lib.fmoe_routing_workspace_bytes(n, e), gate_idx.device)
+        check(lib.fmoe_prune_gate_by_capacity(_ptr(gate_idx), _ptr(out), _ptr(expert_count), n, e, _ptr(ws),
+                                              ws.numel(), _stream(gate_idx)))
+    return out
+
+
+# ---- row permutes -------------------------------------------------------------
+
+def _rows(name, t):
+    _dev(name, t)
+    if t.dim() != 2:
+        raise ValueError(f"{name} must be 2-D [rows, features], got shape {tuple(t.shape)}")
+    return _float_dtype(name, t)
+
+
+def gather_rows(inp, index, n_out=None):
+    """out[r] = inp[index[r]] (zero row where index[r] < 0)."""
+    dt = _rows("inp", inp)
+    _dev("index", index, torch.int64)
+    n_out = index.numel() if n_out is None else n_out
+    out = torch.empty(n_out, inp.shape[1], dtype=inp.dtype, device=inp.device)
+    with torch.cuda.device(inp.device):
+        check(_lib.load().fmoe_gather_rows(_ptr(inp), _ptr(index), _ptr(out), n_out, inp.shape[0], inp.shape[1],
+                                           dt, _stream(inp)))
+    return out
+
+
+def invert_index(pos, n_out):
+    """inverse[pos[i]] = i, -1 elsewhere."""
+    _dev("pos", pos, torch.int64)
+    inv = torch.empty(n_out, dtype=torch.int64, device=pos.device)
+    with torch.cuda.device(pos.device):
+        check(_lib.load().fmoe_invert_index(_ptr(pos), pos.numel(), _ptr(inv), n_out, _stream(pos)))
+    return inv
+
+
+def reduce_slots(inp, slot_to_row, n_tokens, top_k):
+    """out[t] = sum over the token's top_k slots of inp[slot_to_row[slot]]."""
+    dt = _rows("inp", inp)
+    _dev("slot_to_row", slot_to_row, torch.int64)
+    if slot_to_row.numel() != n_tokens * top_k:
+        raise ValueError("slot_to_row must have n_tokens * top_k entries")
+    out = torch.empty(n_tokens, inp.shape[1], dtype=inp.dtype, device=inp.device)
+    with torch.cuda.device(inp.device):
+        check(_lib.load().fmoe_reduce_slots(_ptr(inp), _ptr(slot_to_row), _ptr(out), n_tokens, top_k,
+                                            inp.shape[0], inp.shape[1], dt, _stream(inp)))
+    return out
+
+
+def index_add_rows(inp, index, n_out):
+    """zeros(n_out, d).index_add_(0, index, inp), summed in a fixed order."""
+    dt = _rows("inp", inp)
+    _dev("index", index, torch.int64)
+    if index.numel() != inp.shape[0]:
+        raise ValueError("index must have one entry per row of inp")
+    lib = _lib.load()
+    out = torch.empty(n_out, inp.shape[1], dtype=inp.dtype, device=inp.device)
+    with torch.cuda.device(inp.device):
+        ws = _workspace(lib.fmoe_index_add_workspace_bytes(inp.shape[0], n_out), inp.device)
+        check(lib.fmoe_index_add_rows(_ptr(inp), _ptr(index), _ptr(out), inp.shape[0], n_out, inp.shape[1], dt,
+                                      _ptr(ws), ws.numel(), _stream(inp)))
+    return out
+
+
+# ---- per-expert linear ----------------------------------------------------------
+
+def _check_linear(input_buf, expert_count, weight, bias):
+    dt = _rows("input_buf", input_buf)
+    _dev("weight", weight, input_buf.dtype)
+    if weight.dim() != 3:
+        raise ValueError(f"weight must be [num_expert, out_feat, in_feat], got {tuple(weight.shape)}")
+    n_expert, out_feat, in_feat = weight.shape
+    if input_buf.shape[1] != in_feat:
+        raise ValueError(f"input_buf has {input_buf.shape[1]} features, weight expects {in_feat}")
+    cnt = _host_counts("expert_count", expert_count, n_expert)
+    total = int(cnt.sum())
+    if total != input_buf.shape[0]:
+        raise ValueError(f"expert_count sums to {total} but input_buf has {input_buf.shape[0]} rows")
+    if bias is not None:
+        _dev("bias", bias, input_buf.dtype)
+        if tuple(bias.shape) != (n_expert, out_feat):
+            raise ValueError(f"bias must be [{n_expert}, {out_feat}], got {tuple(bias.shape)}")
+    return dt, cnt, n_expert, out_feat, in_feat
+
+
+def linear_forward(input_buf, expert_count, weight, bias=None):
+    """Y[seg_e] = X[seg_e] @ W_e^T (+ b_e).  fmoe_cuda.linear_forward,
+    cuda/parallel_linear.cu:5-49; ``expert_count`` is a CPU int64 tensor."""
+    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    out = torch.empty(input_buf.shape[0], out_feat, dtype=input_buf.dtype, device=input_buf.device)
+    with torch.cuda.device(input_buf.device):
+        check(_lib.load().fmoe_linear_forward(_ptr(input_buf), _ptr(weight), _ptr(bias), _ptr(out),
+                                              ctypes.c_void_p(cnt.data_ptr()), n_expert, in_feat, out_feat, dt,
+                                              _stream(input_buf)))
+    return out
+
+
+def linear_backward(grad_output_buf, input_buf, expert_count, weight, bias=None):
+    """Returns [grad_input, grad_weight, grad_bias].  fmoe_cuda.linear_backward,
+    cuda/parallel_linear.cu:52-94.  ``grad_bias`` is computed only when ``bias``
+    is given (the reference returns an uninitialised tensor otherwise); without
+    bias it is ``None``."""
+    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    _dev("grad_output_buf", grad_output_buf, input_buf.dtype)
+    if tuple(grad_output_buf.shape) != (input_buf.shape[0], out_feat):
+        raise ValueError(f"grad_output_buf must be [{input_buf.shape[0]}, {out_feat}]")
+    grad_in = torch.empty_like(input_buf)
+    grad_w = torch.empty_like(weight)
+    grad_b = torch.empty(n_expert, out_feat, dtype=input_buf.dtype, device=input_buf.device) \
+        if bias is not None else None
+    with torch.cuda.device(input_buf.device):
+        check(_lib.load().fmoe_linear_backward(_ptr(grad_output_buf), _ptr(input_buf), _ptr(weight), _ptr(grad_in),
+                                               _ptr(grad_w), _ptr(grad_b), ctypes.c_void_p(cnt.data_ptr()),
+                                               n_expert, in_feat, out_feat, dt, _stream(input_buf)))
+    return [grad_in, grad_w, grad_b]
+
+
+# ---- fused expert MLP (chunked, stream-overlapped pipeline) -------------------------
+
+def _mlp_params(w1, b1, w2, b2, activation):
+    dt = _float_dtype("w1", _dev("w1", w1))
+    _dev("w2", w2, w1.dtype)
+    if w1.dim() != 3 or w2.dim() != 3:
+        raise ValueError("w1 / w2 must be [num_expert, out_feat, in_feat]")
+    n_expert, d_hidden, d_model = w1.shape
+    if tuple(w2.shape) != (n_expert, d_model, d_hidden):
+        raise ValueError(f"w2 must be [{n_expert}, {d_model}, {d_hidden}], got {tuple(w2.shape)}")
+    for name, b, width in (("b1", b1, d_hidden), ("b2", b2, d_model)):
+        if b is not None:
+            _dev(name, b, w1.dtype)
+            if tuple(b.shape) != (n_expert, width):
+                raise ValueError(f"{name} must be [{n_expert}, {width}]")
+    if dt == _lib.F64:
+        raise TypeError("the fused expert MLP supports float32, bfloat16 and float16")
+    if activation not in (_lib.ACT_NONE, _lib.ACT_RELU, _lib.ACT_GELU):
+        raise ValueError(f"unknown activation code {activation}")
+    prm = _lib.MlpParams(w1.data_ptr(), b1.data_ptr() if b1 is not None else None, w2.data_ptr(),
+                         b2.data_ptr() if b2 is not None else None, n_expert, d_model, d_hidden, dt, activation)
+    return prm, n_expert, d_model, d_hidden
+
+
+def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k, activation, n_chunks):
+    """scatter -> Linear -> activation -> Linear -> gather as one pipelined call.
+    Returns ``(out [N*top_k, d], buf_in, buf_pre or None, buf_mid)``; the three
+    buffers are what the backward needs."""
+    prm, n_expert, d_model, d_hidden = _mlp_params(w1, b1, w2, b2, activation)
+    _dev("inp", inp, w1.dtype)
+    _dev("pos", pos, torch.int64)
+    _dev("slot_to_row", slot_to_row, torch.int64)
+    if inp.dim() != 2 or inp.shape[1] != d_model:
+        raise ValueError(f"inp must be [n_tokens, {d_model}]")
+    n_tokens, n_rows = inp.shape[0], pos.numel()
+    if slot_to_row.numel() != n_tokens * top_k:
+        raise ValueError("slot_to_row must have n_tokens * top_k entries")
+    cnt = _host_counts("expert_count", expert_count, n_expert)
+    new = lambda r, c: torch.empty(r, c, dtype=inp.dtype, device=inp.device)
+    buf_in, buf_mid, buf_out = new(n_rows, d_model), new(n_rows, d_hidden), new(n_rows, d_model)
+    buf_pre = new(n_rows, d_hidden) if activation == _lib.ACT_GELU else None
+    out = new(n_tokens * top_k, d_model)
+    with torch.cuda.device(inp.device):
+        check(_lib.load().fmoe_fused_mlp_forward(
+            ctypes.byref(prm), _ptr(inp), _ptr(pos), _ptr(slot_to_row), ctypes.c_void_p(cnt.data_ptr()),
+            n_tokens, top_k, n_rows, _ptr(buf_in), _ptr(buf_pre), _ptr(buf_mid), _ptr(buf_out), _ptr(out),
+            n_chunks, _stream(inp)))
+    return out, buf_in, buf_pre, buf_mid
+
+
+def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid,
+                       n_tokens, top_k, activation, n_chunks):
+    """Backward of :func:`fused_mlp_forward`.  Returns
+    ``(grad_inp, grad_w1, grad_b1, grad_w2, grad_b2)`` (bias grads ``None``
+    without biases).  For ReLU the post-activation buffer doubles as the
+    pre-activation (same sign pattern)."""
+    prm, n_expert, d_model, d_hidden = _mlp_params(w1, b1, w2, b2, activation)
+    _dev("grad_out", grad_out, w1.dtype)
+    if tuple(grad_out.shape) != (n_tokens * top_k, d_model):
+        raise ValueError(f"grad_out must be [{n_tokens * top_k}, {d_model}]")
+    n_rows = pos.numel()
+    cnt = _host_counts("expert_count", expert_count, n_expert)
+    pre = buf_pre if buf_pre is not None else buf_mid
+    dev, dty = grad_out.device, grad_out.dtype
+    new = lambda *s: torch.empty(*s, dtype=dty, device=dev)
+    g_out, g_mid, g_in = new(n_rows, d_model), new(n_rows, d_hidden), new(n_rows, d_model)
+    grad_inp = new(n_tokens, d_model)
+    grad_w1, grad_w2 = torch.empty_like(w1), torch.empty_like(w2)
+    grad_b1 = torch.empty_like(b1) if b1 is not None else None
+    grad_b2 = torch.empty_like(b2) if b2 is not None else None
+    with torch.cuda.device(dev):
+        check(_lib.load().fmoe_fused_mlp_backward(
+            ctypes.byref(prm), _ptr(grad_out), _ptr(pos), _ptr(slot_to_row), ctypes.c_void_p(cnt.data_ptr()),
+            n_tokens, top_k, n_rows, _ptr(buf_in), _ptr(pre), _ptr(buf_mid), _ptr(g_out), _ptr(g_mid), _ptr(g_in),
+            _ptr(grad_inp), _ptr(grad_w1), _ptr(grad_b1), _ptr(grad_w2), _ptr(grad_b2), n_chunks,
+            _stream(grad_out)))
+    return grad_inp, grad_w1, grad_b1, grad_w2, grad_b2
+
+
+def _fuse_chunks():
+    import os
+    return max(1, int(os.environ.get("FMOE_FUSE_GRAN", "4")))
+
+
+def _unpack_params(params, has_bias):
+    expert = params[0][0]
+    if has_bias:
+        w1, b1, w2, b2 = expert
+    else:
+        w1, w2 = expert[0], expert[len(expert) // 2]
+        b1 = b2 = None
+    return w1, b1, w2, b2
+
+
+def fused_forward(input_buf, params, local_expert_count, global_expert_count, stored_models,
+                  global_batch_size, n_workers, has_bias):
+    """fmoe_cuda.fused_forward (cuda/fused_compute.cu:12-62) for one worker:
+    ``input_buf`` is already expert-sorted, the activation is ReLU as in the
+    reference kernel (cuda/fused_compute.cuh:20-44).  Returns
+    ``[output_buf, global_input_buf, global_middle_buf, global_output_buf]``."""
+    if n_workers != 1:
+        raise NotImplementedError("fused_forward: one worker only")
+    w1, b1, w2, b2 = _unpack_params(params, has_bias)
+    rows = input_buf.shape[0]
+    ident = torch.arange(rows, dtype=torch.int64, device=input_buf.device)
+    out, buf_in, _pre, buf_mid = fused_mlp_forward(input_buf.contiguous(), ident, ident, global_expert_count,
+                                                   w1, b1, w2, b2, 1, _lib.ACT_RELU, _fuse_chunks())
+    return [out, buf_in, buf_mid, out]
+
+
+def fused_backward(input_buf, params, middle_buf, output_buf, grad_out, local_expert_count,
+                   global_expert_count, inp, stored_models, global_batch_size, buf_batch_size,
+                   n_workers, has_bias):
+    """fmoe_cuda.fused_backward (cuda/fused_compute.cu:64-131) for one worker.
+    Returns ``[grad_in]`` and, like the reference, leaves the weight gradients
+    in ``param.grad`` -- ADDED to an existing ``.grad`` (the reference overwrites
+    it on its first pipeline step, cuda/fused_compute.cuh:123)."""
+    if n_workers != 1:
+        raise NotImplementedError("fused_backward: one worker only")
+    w1, b1, w2, b2 = _unpack_params(params, has_bias)
+    rows = input_buf.shape[0]
+    ident = torch.arange(rows, dtype=torch.int64, device=input_buf.device)
+    grad_in, gw1, gb1, gw2, gb2 = fused_mlp_backward(
+        grad_out.contiguous(), ident, ident, global_expert_count, w1, b1, w2, b2, input_buf, None, middle_buf,
+        rows, 1, _lib.ACT_RELU, _fuse_chunks())
+    for prm, g in ((w1, gw1), (b1, gb1), (w2, gw2), (b2, gb2)):
+        if prm is None:
+            continue
+        if prm.grad is None:
+            prm.grad = g
+        else:
+            prm.grad.add_(g)
+    return [grad_in]

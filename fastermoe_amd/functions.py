@@ -1,0 +1,193 @@
+r"""Autograd Functions and routing helpers of the MoE layer, with the interface of
+the reference's ``fmoe.functions`` (fmoe/functions.py), on top of
+:mod:`fastermoe_amd.fmoe_native`.
+
+Single worker only: ``world_size > 1`` (token all-to-all, dynamic shadowing) is
+outside this package and raises ``NotImplementedError``.
+"""
+import torch
+from torch.autograd import Function
+
+from . import fmoe_native
+
+
+def _single_worker(world_size, what):
+    if world_size != 1:
+        raise NotImplementedError(
+            f"{what}: world_size={world_size}; this package implements the single-GPU "
+            "path only (no global exchange, no dynamic shadowing)")
+
+
+def ensure_comm(t, comm):
+    """fmoe/functions.py:14-17 binds an NCCL communicator; nothing to do for one worker."""
+    return None
+
+
+def _route(gate, num_expert, world_size):
+    """(pos, counts, slot_to_row): one fused routing call and ONE device-to-host
+    read (the counts), instead of the histogram / cumsum / ``.item()`` /
+    placement sequence of fmoe/functions.py:19-42."""
+    _single_worker(world_size, "count_by_gate")
+    with torch.no_grad():
+        counts, pos_buf, slot_to_row = fmoe_native.route(gate.contiguous(), num_expert)
+        counts_cpu = counts.cpu()
+        pos = pos_buf[: int(counts_cpu.sum())]
+    return pos, counts, counts_cpu, slot_to_row
+
+
+def count_by_gate(gate, num_expert, world_size, require_pos=True):
+    """fmoe/functions.py:19-42.  Returns ``(pos, local_expert_count,
+    all_expert_count, global_expert_count, all_global_expert_count)``; with one
+    worker the four count tensors are the same int64 ``[num_expert]`` tensor."""
+    _single_worker(world_size, "count_by_gate")
+    with torch.no_grad():
+        if not require_pos:
+            cnt32 = torch.zeros(num_expert, device=gate.device, dtype=torch.int32)
+            fmoe_native.expert_count(gate.contiguous(), cnt32)
+            counts = cnt32.long()
+            pos = None
+        else:
+            pos, counts, _, _ = _route(gate, num_expert, world_size)
+    return pos, counts, counts, counts, counts
+
+
+def _prepare_forward_ex(gate, num_expert, world_size):
+    pos, counts, counts_cpu, slot_to_row = _route(gate, num_expert, world_size)
+    return (pos, counts_cpu, counts_cpu, counts_cpu, counts_cpu, counts_cpu.clone()), slot_to_row
+
+
+def prepare_forward(gate, num_expert, world_size):
+    r"""fmoe/functions.py:45-69: ``(pos, local_expert_count, global_expert_count,
+    all_expert_count, all_global_expert_count, fwd_expert_count)`` with ``pos`` on
+    the device and the counts on the CPU."""
+    return _prepare_forward_ex(gate, num_expert, world_size)[0]
+
+
+def _local_scatter(inp, pos):
+    """fmoe/functions.py:72-74 (index_select)."""
+    return fmoe_native.gather_rows(inp.contiguous(), pos)
+
+
+def _local_gather(inp, pos, out_batch_size, maybe_overlap=True):
+    """fmoe/functions.py:77-84: zero-fill then index_add_ (``maybe_overlap``) or
+    index_copy_."""
+    inp = inp.contiguous()
+    if maybe_overlap:
+        return fmoe_native.index_add_rows(inp, pos, out_batch_size)
+    inverse = fmoe_native.invert_index(pos, out_batch_size)
+    return fmoe_native.gather_rows(inp, inverse)
+
+
+class MOECache(Function):
+    r"""fmoe/functions.py:122-194.  The reference decides here which experts to
+    shadow on other workers and raises for one worker; with one worker there is
+    nothing to shadow, so this is the identity: ``models = [[experts]]``,
+    ``stored_models`` all False, counts unchanged."""
+
+    @staticmethod
+    def forward(ctx, inp, all_expert_count, all_global_expert_count, local_expert_count,
+                global_expert_count, fwd_expert_count, policy_fn, experts, batch_size, d_model,
+                topk, num_expert, world_size, fused):
+        _single_worker(world_size, "MOECache")
+        stored_models = torch.zeros(world_size * num_expert, dtype=torch.bool)
+        models = [[experts]] if fused else [experts]
+        ctx.mark_non_differentiable(stored_models, fwd_expert_count)
+        return inp.view_as(inp), models, stored_models, fwd_expert_count, int(fwd_expert_count.sum().item())
+
+    @staticmethod
+    def backward(ctx, grad_inp, *unused):
+        return (grad_inp,) + (None,) * 13
+
+
+class MOEScatter(Function):
+    r"""Token rows -> expert-sorted rows (fmoe/functions.py:196-248).  ``pos`` is
+    the token index of every sorted row (``pos // top_k``).  The two trailing
+    arguments are optional extras: given ``slot_to_row`` and ``top_k`` the
+    backward sums each token's ``top_k`` rows directly instead of going through
+    the general index-add."""
+
+    @staticmethod
+    def forward(ctx, inp, pos, local_expert_count, global_expert_count, stored_models,
+                fwd_batch_size, world_size, slot_to_row=None, top_k=None):
+        _single_worker(world_size, "MOEScatter")
+        buf = _local_scatter(inp, pos)
+        ctx.moe_args = inp.shape[0], top_k
+        ctx.save_for_backward(pos, slot_to_row)
+        return buf
+
+    @staticmethod
+    def backward(ctx, grad_buf):
+        pos, slot_to_row = ctx.saved_tensors
+        n_tokens, top_k = ctx.moe_args
+        grad_buf = grad_buf.contiguous()
+        if slot_to_row is not None:
+            grad_in = fmoe_native.reduce_slots(grad_buf, slot_to_row, n_tokens, top_k)
+        else:
+            grad_in = _local_gather(grad_buf, pos, n_tokens)
+        return grad_in, None, None, None, None, None, None, None, None
+
+
+class MOELinear(Function):
+    r"""Per-expert linear over expert-sorted rows (fmoe/functions.py:251-275)."""
+
+    @staticmethod
+    def forward(ctx, global_input_buf, fwd_expert_count, weight, bias=None):
+        global_input_buf = global_input_buf.contiguous()
+        out = fmoe_native.linear_forward(global_input_buf, fwd_expert_count, weight, bias)
+        ctx.save_for_backward(global_input_buf, fwd_expert_count, weight, bias)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        input_buf, fwd_expert_count, weight, bias = ctx.saved_tensors
+        grad_in, grad_w, grad_b = fmoe_native.linear_backward(
+            grad_out.contiguous(), input_buf, fwd_expert_count, weight, bias)
+        return grad_in, None, grad_w, grad_b
+
+
+class MOEGather(Function):
+    r"""Expert-sorted rows -> slot order, zero rows for dropped slots
+    (fmoe/functions.py:278-330).  ``slot_to_row`` (optional extra) is the inverse
+    of ``pos``; without it the inverse is rebuilt from ``pos``."""
+
+    @staticmethod
+    def forward(ctx, global_output_buf, pos, local_expert_count, global_expert_count,
+                stored_models, local_batch_size, world_size, slot_to_row=None):
+        _single_worker(world_size, "MOEGather")
+        buf = global_output_buf.contiguous()
+        if slot_to_row is None:
+            slot_to_row = fmoe_native.invert_index(pos, local_batch_size)
+        out = fmoe_native.gather_rows(buf, slot_to_row, local_batch_size)
+        ctx.save_for_backward(pos)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (pos,) = ctx.saved_tensors
+        return _local_scatter(grad_out, pos), None, None, None, None, None, None, None
+
+
+class AllGather(Function):
+    r"""fmoe/functions.py:333-349 (model-parallel group); one worker only."""
+
+    @staticmethod
+    def forward(ctx, inp, rank, world_size, group):
+        _single_worker(world_size, "AllGather")
+        return inp.view_as(inp)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        return grad_out, None, None, None
+
+
+class Slice(Function):
+    r"""fmoe/functions.py:352-375 (model-parallel group); one worker only."""
+
+    @staticmethod
+    def forward(ctx, inp, rank, world_size, group):
+        _single_worker(world_size, "Slice")
+        return inp.view_as(inp)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        return grad_out, None, None, None

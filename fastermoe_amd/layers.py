@@ -1,0 +1,217 @@
+r"""MoE modules with the constructor and forward signatures of the reference's
+``fmoe.layers`` (fmoe/layers.py), for one worker."""
+import math
+import os
+
+import torch
+import torch.nn as nn
+
+from .functions import (AllGather, MOECache, MOEGather, MOELinear, MOEScatter, Slice,
+                        _prepare_forward_ex, ensure_comm)
+from .gates import NaiveGate
+
+
+class FMoELinear(nn.Module):
+    r"""``num_expert`` linear layers applied to consecutive row segments of the
+    input in one grouped GEMM (fmoe/layers.py:16-67).  ``weight`` is
+    ``[num_expert, out_feat, in_feat]``, ``bias`` ``[num_expert, out_feat]``."""
+
+    def __init__(self, num_expert: int, in_feat: int, out_feat: int, bias: bool = True, rank: int = 0):
+        super().__init__()
+        self.num_expert = num_expert
+        self.in_feat = in_feat
+        self.out_feat = out_feat
+        self.rank = rank
+        self.weight = nn.Parameter(torch.empty(num_expert, out_feat, in_feat))
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(num_expert, out_feat))
+        else:
+            self.register_parameter("bias", None)
+        self.reset_parameters()
+
+    def forward(self, inp, fwd_expert_count):
+        return MOELinear.apply(inp, fwd_expert_count, self.weight, self.bias)
+
+    def extra_repr(self) -> str:
+        return "num_expert={}, in_features={}, out_features={}, bias={}, rank={}".format(
+            self.num_expert, self.in_feat, self.out_feat, self.bias is not None, self.rank)
+
+    def reset_parameters(self):
+        # Kaiming-uniform over the whole 3-D tensor, bias left at zero
+        # (fmoe/layers.py:62-67)
+        torch.nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+
+
+def mark_module_parallel_comm(module, comm):
+    r"""Tags every parameter with the data-parallel group it is synchronised in
+    (fmoe/layers.py:70-76)."""
+    for p in module.parameters():
+        setattr(p, "dp_comm", comm)
+
+
+def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_expert, world_size,
+                                 fused, enable_fuse=False):
+    r"""Route, scatter, run the experts, gather (fmoe/layers.py:79-149).  Returns
+    ``(rows in slot order [N*top_k, d], stored_models)``."""
+    from .fused_functions import MOEForward
+
+    (pos, local_expert_count, global_expert_count, all_expert_count, all_global_expert_count,
+     fwd_expert_count), slot_to_row = _prepare_forward_ex(gate, num_expert, world_size)
+
+    topk = gate.shape[1] if gate.dim() == 2 else 1
+    out_batch_size = inp.shape[0] * topk
+
+    inp, models, stored_models, fwd_expert_count, fwd_batch_size = MOECache.apply(
+        inp,
+        all_expert_count.view(world_size, world_size, num_expert),
+        all_global_expert_count.view(world_size, world_size, num_expert),
+        local_expert_count.view(world_size, num_expert),
+        global_expert_count.view(world_size, num_expert),
+        fwd_expert_count, policy_fn, experts, inp.shape[0], inp.shape[1], topk, num_expert,
+        world_size, fused)
+
+    if enable_fuse:
+        x = MOEForward.apply(inp, models, pos // topk, pos, local_expert_count, global_expert_count,
+                             stored_models, fwd_batch_size, out_batch_size, world_size, slot_to_row)
+        return x, stored_models
+
+    # ZeroGate hands back N*top_k indices as a 1-D tensor, so the slot count can
+    # exceed the token count; the per-token reduction only applies when it does not.
+    per_token = slot_to_row if slot_to_row.numel() == inp.shape[0] * topk else None
+    x = MOEScatter.apply(inp, pos // topk, local_expert_count, global_expert_count, stored_models,
+                         fwd_batch_size, world_size, per_token, topk)
+    x = expert_fn(x, models, fwd_expert_count, num_expert)
+    x = MOEGather.apply(x, pos, local_expert_count, global_expert_count, stored_models,
+                        out_batch_size, world_size,
+                        slot_to_row if slot_to_row.numel() == out_batch_size else None)
+    return x, stored_models
+
+
+class FMoE(nn.Module):
+    r"""General MoE layer (fmoe/layers.py:151-326).
+
+    * ``num_expert``: experts on this worker; ``world_size`` must be 1 here.
+    * ``top_k``: experts per token; ``gate``: a class from :mod:`fastermoe_amd.gates`.
+    * ``expert``: a module class (or list of classes) instantiated per expert and
+      called on row slices; ``None`` means the subclass provides a fused
+      ``self.experts`` taking ``(rows, fwd_expert_count)``.
+    * ``enable_fuse`` (or ``FMOE_ENABLE_FUSE=1``): run scatter, the expert MLP and
+      gather as one chunked, stream-overlapped pipeline.
+    """
+
+    def __init__(self, num_expert=32, d_model=1024, world_size=1, mp_group=None, moe_group=None,
+                 top_k=2, gate=NaiveGate, expert=None, gate_hook=None, policy_fn=None, mask=None,
+                 mask_dict=None, enable_fuse=False):
+        super().__init__()
+        if world_size != 1:
+            raise NotImplementedError("fastermoe_amd implements the single-GPU path: world_size must be 1")
+        self.num_expert = num_expert
+        self.d_model = d_model
+        self.world_size = world_size
+        self.mp_group = mp_group
+        if mp_group is None:
+            self.mp_size = 1
+            self.mp_rank = 0
+        else:
+            self.mp_size = mp_group.size()
+            self.mp_rank = mp_group.rank()
+            if self.mp_size != 1:
+                raise NotImplementedError("model-parallel groups larger than 1 are not supported")
+        self.top_k = top_k
+        if type(expert) is list:
+            self.experts = nn.ModuleList([e(d_model) for e in expert])
+            self.experts_fused = False
+            self.num_expert = num_expert = len(expert)
+        elif expert is not None:
+            self.experts = nn.ModuleList([expert(d_model) for _ in range(num_expert)])
+            self.experts_fused = False
+        else:
+            self.experts_fused = True
+        self.gate = gate(d_model, num_expert, world_size, top_k)
+        if hasattr(self.gate, "stored_models"):
+            self.gate.policy_fn = policy_fn
+        self.gate_hook = gate_hook
+        self.mask = mask
+        self.mask_dict = mask_dict
+        self.moe_group = moe_group
+
+        if os.environ.get("FMOE_ENABLE_FUSE", "0") == "1":
+            enable_fuse = True
+        self.enable_fuse = enable_fuse
+        if enable_fuse:
+            assert self.experts_fused
+        self.policy_fn = policy_fn
+
+    def expert_fn(self, inp, models, fwd_expert_count, num_expert):
+        r"""Runs the experts on expert-sorted rows (fmoe/layers.py:222-255): the
+        fused expert module in one call, or one module per row slice."""
+        res = []
+        input_ptr = 0
+        for j, counts in enumerate(fwd_expert_count.view(-1, num_expert)):
+            size = int(counts.sum().item())
+            node_inp = inp[input_ptr:input_ptr + size]
+            input_ptr += size
+            experts = models[j]
+            if not experts:
+                if counts.any():
+                    raise ValueError(f"Experts is {experts} yet counts is {counts}")
+                continue
+            if self.experts_fused:
+                res.append(experts[0](node_inp, counts))
+                continue
+            outputs = []
+            base_idx = 0
+            for i in range(self.num_expert):
+                batch_size = int(counts[i].item())
+                outputs.append(experts[i](node_inp[base_idx:base_idx + batch_size]))
+                base_idx += batch_size
+            res.append(torch.cat(outputs, dim=0))
+        return torch.cat(res, dim=0)
+
+    def mark_parallel_comm(self, expert_dp_comm="none"):
+        r"""fmoe/layers.py:257-270."""
+        if self.experts is not None:
+            if isinstance(self.experts, list):
+                for e in self.experts:
+                    mark_module_parallel_comm(e, expert_dp_comm)
+            else:
+                mark_module_parallel_comm(self.experts, expert_dp_comm)
+        mark_module_parallel_comm(self.gate, "moe")
+
+    def forward(self, inp):
+        r"""Gate, route through the experts, and combine each token's ``top_k``
+        expert outputs with the gate scores (fmoe/layers.py:272-326)."""
+        if self.world_size > 1:
+            ensure_comm(inp, self.moe_group)
+        if self.mp_size > 1:
+            inp = Slice.apply(inp, self.mp_rank, self.mp_size, self.mp_group)
+
+        gate_top_k_idx, gate_score = self.gate(inp)
+        if self.gate_hook is not None:
+            self.gate_hook(gate_top_k_idx, gate_score, None)
+
+        masked = self.mask is not None and self.mask_dict is not None
+        if masked:
+            mask = self.mask.view(-1)
+            inp = inp[mask == 0, :]
+            gate_top_k_idx = gate_top_k_idx[mask == 0, :]
+
+        fwd, _stored_models = _fmoe_general_global_forward(
+            inp, gate_top_k_idx, self.expert_fn, self.policy_fn, self.experts, self.num_expert,
+            self.world_size, self.experts_fused, self.enable_fuse)
+
+        if masked:
+            fwd = fwd.view(-1, self.top_k, self.d_model)
+            x = torch.zeros(mask.shape[0], self.top_k, self.d_model, device=fwd.device, dtype=fwd.dtype)
+            x[mask == 0] = fwd
+            for k, v in self.mask_dict.items():
+                x[mask == k] = v
+        else:
+            x = fwd.view(-1, self.top_k, self.d_model)
+
+        gate_score = gate_score.view(x.shape[0], 1, self.top_k)
+        x = torch.bmm(gate_score, x).reshape(-1, self.d_model)
+
+        if self.mp_size > 1:
+            x = AllGather.apply(x, self.mp_rank, self.mp_size, self.mp_group)
+        return x

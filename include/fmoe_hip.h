@@ -1,0 +1,222 @@
+/*
+ * fmoe_hip.h -- C ABI of libfmoe_hip.so, the gfx950 (MI355X) kernels behind the
+ * fmoe Python API's single-GPU MoE path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     all work is enqueued on it and nothing synchronises with the host;
+ *   - every entry point returns 0 on success and a negative FMOE_E* code on
+ *     failure; fmoe_last_error() then holds a message for the calling thread;
+ *   - inputs are borrowed, outputs are caller-allocated, nothing is freed here;
+ *   - tensors are dense row-major.
+ *
+ * Each entry point names the reference interface (thu-pacman/FasterMoE) it
+ * stands in for.
+ */
+#ifndef FMOE_HIP_H
+#define FMOE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FMOE_OK 0
+#define FMOE_EINVAL (-1)    /* bad argument (shape, alignment, dtype, NULL) */
+#define FMOE_ELIMIT (-2)    /* size beyond what the kernels support */
+#define FMOE_EHIP (-3)      /* a HIP runtime call failed */
+#define FMOE_EWORKSPACE (-4) /* workspace missing or too small */
+
+/* element types of activation / weight tensors */
+#define FMOE_F32 0
+#define FMOE_BF16 1
+#define FMOE_F16 2
+#define FMOE_F64 3
+
+/* activation between the two expert linears of the fused MLP */
+#define FMOE_ACT_NONE 0
+#define FMOE_ACT_RELU 1
+#define FMOE_ACT_GELU 2 /* exact erf form, torch.nn.GELU() default */
+
+const char *fmoe_last_error(void);
+int fmoe_abi_version(void);
+
+/* ---- routing bookkeeping ------------------------------------------------ */
+
+/* expert_count[e] += #{i : gate_idx[i] == e}; entries outside [0, n_expert)
+ * (the -1 of dropped slots) are skipped.  The caller zero-fills.
+ * Replaces fmoe_cuda_expert_count_impl, cuda/local_exchange.cuh:63-71
+ * (bound as fmoe_cuda.expert_count, cuda/fmoe_cuda.cpp:119). */
+int fmoe_expert_count(const int64_t *gate_idx, int32_t *expert_count,
+                      int64_t n_slots, int64_t n_expert, void *stream);
+
+/* Bytes of scratch the rank-based routing entry points below need. */
+int64_t fmoe_routing_workspace_bytes(int64_t n_slots, int64_t n_expert);
+
+/* Counting-sort placement.  cum_count enters as the int32 inclusive cumsum of
+ * the expert counts and leaves as the exclusive one; pos[cum[e]-n_e .. cum[e])
+ * receives the flat slot indices routed to expert e in DESCENDING index order
+ * (what the reference kernel yields when its threads run one at a time in
+ * ascending index).  pos holds n_pos entries; rows beyond it are not written.
+ * Replaces fmoe_cuda_assign_pos_impl,
+ * cuda/local_exchange.cuh:18-27 (fmoe_cuda.assign_pos, cuda/fmoe_cuda.cpp:120). */
+int fmoe_assign_pos(int32_t *cum_count, const int64_t *gate, int64_t *pos,
+                    int64_t n_pos, int64_t n_slots, int64_t n_expert,
+                    void *workspace, int64_t workspace_bytes, void *stream);
+
+/* One call for count + cumsum + placement (what fmoe/functions.py:19-42 does
+ * with two kernels, a torch.cumsum and a host read in between):
+ *   expert_count [n_expert] int64  <- histogram (overwritten, not accumulated)
+ *   pos          [n_slots]  int64  <- first sum(expert_count) entries as in
+ *                                     fmoe_assign_pos, the rest untouched
+ *   slot_to_row  [n_slots]  int64  <- inverse of pos: row of each slot in the
+ *                                     expert-sorted order, -1 for dropped slots
+ *                                     (may be NULL) */
+int fmoe_route(const int64_t *gate, int64_t n_slots, int64_t n_expert,
+               int64_t *expert_count, int64_t *pos, int64_t *slot_to_row,
+               void *workspace, int64_t workspace_bytes, void *stream);
+
+/* ---- capacity balancing ------------------------------------------------- */
+
+/* eca[w,e] = share of cap[e] granted to worker w, workers served in ascending
+ * order; cap[e] is decremented by every proposal.  Replaces
+ * fmoe_cuda_limit_by_capacity_impl, cuda/balancing.cuh:23-31
+ * (fmoe_cuda.limit_by_capacity, cuda/fmoe_cuda.cpp:125). */
+int fmoe_limit_by_capacity(const int64_t *ec, int32_t *cap, int64_t *eca,
+                           int64_t n_expert, int64_t n_worker, void *stream);
+
+/* new_gate_idx[i] = gate_idx[i] if fewer than ec[gate_idx[i]] slots with a
+ * lower flat index chose the same expert, else -1.  ec[e] is decremented once
+ * per slot that names e.  Slots already -1 stay -1.  Replaces
+ * fmoe_cuda_prune_gate_by_capacity_impl, cuda/balancing.cuh:48-58
+ * (fmoe_cuda.prune_gate_by_capacity, cuda/fmoe_cuda.cpp:126). */
+int fmoe_prune_gate_by_capacity(const int64_t *gate_idx, int64_t *new_gate_idx,
+                                int32_t *ec, int64_t n_slots, int64_t n_expert,
+                                void *workspace, int64_t workspace_bytes,
+                                void *stream);
+
+/* ---- local scatter / gather (row permutes) ------------------------------ */
+
+/* out[r,:] = index[r] >= 0 ? inp[index[r],:] : 0   for r in [0, n_out).
+ * Replaces _local_scatter = torch.index_select, fmoe/functions.py:72-74. */
+int fmoe_gather_rows(const void *inp, const int64_t *index, void *out,
+                     int64_t n_out, int64_t n_inp, int64_t row_elems, int dtype,
+                     void *stream);
+
+/* inverse[0..n_out) = -1, then inverse[pos[i]] = i for i in [0, n_pos).
+ * With it, the zero-fill + index_copy_ of fmoe/functions.py:77-84
+ * (maybe_overlap=False) is one fmoe_gather_rows(inp, inverse, out). */
+int fmoe_invert_index(const int64_t *pos, int64_t n_pos, int64_t *inverse,
+                      int64_t n_out, void *stream);
+
+/* out[t,:] = sum_{j<top_k} rows inp[slot_to_row[t*top_k+j],:] (entries < 0
+ * contribute nothing), summed in fp32 in ascending j.  The atomics-free form of
+ * zeros().index_add_(pos // top_k), fmoe/functions.py:77-82, when the index is
+ * known to be slot positions. */
+int fmoe_reduce_slots(const void *inp, const int64_t *slot_to_row, void *out,
+                      int64_t n_tokens, int64_t top_k, int64_t n_inp,
+                      int64_t row_elems, int dtype, void *stream);
+
+/* General out = zeros(n_out, row).index_add_(0, index, inp) with n_in source
+ * rows (fmoe/functions.py:77-82, maybe_overlap=True), summed in fp32 in
+ * ascending source row, so the result does not depend on scheduling.
+ * workspace: fmoe_index_add_workspace_bytes(n_in, n_out). */
+int64_t fmoe_index_add_workspace_bytes(int64_t n_in, int64_t n_out);
+int fmoe_index_add_rows(const void *inp, const int64_t *index, void *out,
+                        int64_t n_in, int64_t n_out, int64_t row_elems,
+                        int dtype, void *workspace, int64_t workspace_bytes,
+                        void *stream);
+
+/* ---- per-expert linear (one grouped GEMM over ragged row segments) ------ */
+
+/* y[seg_e,:] = x[seg_e,:] . w[e]^T (+ bias[e]); seg_e are consecutive row
+ * ranges of lengths expert_count_host[e].  x [S,in], w [E,out,in],
+ * bias [E,out] or NULL, y [S,out].  Replaces fmoe_cuda_linear_forward_impl,
+ * cuda/parallel_linear.cuh:55-88 (fmoe_cuda.linear_forward). */
+int fmoe_linear_forward(const void *x, const void *w, const void *bias, void *y,
+                        const int64_t *expert_count_host, int64_t n_expert,
+                        int64_t in_feat, int64_t out_feat, int dtype,
+                        void *stream);
+
+/* grad_x[seg_e,:] = grad_y[seg_e,:] . w[e];  grad_w[e] = grad_y[seg_e]^T . x[seg_e]
+ * (zeros for an empty expert);  grad_b[e] = column sums of grad_y[seg_e] when
+ * grad_b != NULL.  Replaces fmoe_cuda_linear_backward_impl,
+ * cuda/parallel_linear.cuh:90-161 (fmoe_cuda.linear_backward). */
+int fmoe_linear_backward(const void *grad_y, const void *x, const void *w,
+                         void *grad_x, void *grad_w, void *grad_b,
+                         const int64_t *expert_count_host, int64_t n_expert,
+                         int64_t in_feat, int64_t out_feat, int dtype,
+                         void *stream);
+
+/* ---- fused expert MLP, chunked pipeline at world_size 1 ----------------- */
+
+typedef struct fmoe_mlp_params {
+    const void *w1;   /* [E, d_hidden, d_model] */
+    const void *b1;   /* [E, d_hidden] or NULL  */
+    const void *w2;   /* [E, d_model, d_hidden] */
+    const void *b2;   /* [E, d_model] or NULL   */
+    int64_t n_expert, d_model, d_hidden;
+    int dtype;        /* FMOE_F32 / FMOE_BF16 / FMOE_F16 */
+    int activation;   /* FMOE_ACT_* */
+} fmoe_mlp_params;
+
+/* Forward of scatter -> Linear -> act -> Linear -> gather over `n_chunks`
+ * contiguous chunks of the expert-sorted rows, chunk c+1's scatter and chunk
+ * c-1's gather running beside chunk c's GEMMs on the library's own streams,
+ * chained by events to `stream` (fork at entry, join at exit).
+ *   inp        [n_tokens, d_model]
+ *   pos        [n_rows] int64   flat slot of every expert-sorted row
+ *   slot_to_row[n_tokens*top_k] int64 (inverse of pos, -1 = dropped)
+ *   buf_in     [n_rows, d_model]   scattered input  (kept for backward)
+ *   buf_pre    [n_rows, d_hidden]  pre-activation   (kept for backward)
+ *   buf_mid    [n_rows, d_hidden]  post-activation  (kept for backward)
+ *   buf_out    [n_rows, d_model]   expert output
+ *   out        [n_tokens*top_k, d_model]  zero rows for dropped slots
+ * Replaces fmoe_cuda_fused_forward_impl at one worker,
+ * cuda/fused_compute.cuh:250-388 (fmoe_cuda.fused_forward) together with the
+ * _local_scatter/_local_gather around it, fmoe/fused_functions.py:22-32. */
+int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
+                           const int64_t *pos, const int64_t *slot_to_row,
+                           const int64_t *expert_count_host, int64_t n_tokens,
+                           int64_t top_k, int64_t n_rows, void *buf_in,
+                           void *buf_pre, void *buf_mid, void *buf_out,
+                           void *out, int n_chunks, void *stream);
+
+/* Backward of the same pipeline.  grad_out [n_tokens*top_k, d_model].
+ * Scratch (caller-allocated): g_out [n_rows,d_model], g_mid [n_rows,d_hidden],
+ * g_in [n_rows,d_model].  Results: grad_inp [n_tokens,d_model], grad_w1/2,
+ * grad_b1/2 (bias grads may be NULL).  Weight grads of an expert split across
+ * chunks accumulate chunk by chunk (cuda/fused_compute.cuh:123: beta_weight).
+ * Replaces fmoe_cuda_fused_backward_impl at one worker,
+ * cuda/fused_compute.cuh:391-542 (fmoe_cuda.fused_backward). */
+int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *grad_out,
+                            const int64_t *pos, const int64_t *slot_to_row,
+                            const int64_t *expert_count_host, int64_t n_tokens,
+                            int64_t top_k, int64_t n_rows, const void *buf_in,
+                            const void *buf_pre, const void *buf_mid,
+                            void *g_out, void *g_mid, void *g_in,
+                            void *grad_inp, void *grad_w1, void *grad_b1,
+                            void *grad_w2, void *grad_b2, int n_chunks,
+                            void *stream);
+
+/* ---- per-launch timing of the library's kernels (off by default) ------- */
+
+/* Kernel classes, in the order of the arrays fmoe_profile_collect fills:
+ * 0 grouped GEMM forward, 1 grouped GEMM data-grad, 2 grouped GEMM weight-grad
+ * (work = flop); 3 bias grad, 4 gather rows, 5 scatter rows, 6 reduce slots,
+ * 7 index add (work = algorithmic bytes).  No counterpart in the reference
+ * (its cuda/utils/timer.hh is commented out); used by bench.py to time each
+ * kernel with HIP events on the stream it is launched on. */
+int fmoe_profile_enable(int on);
+int fmoe_profile_classes(void);
+/* Synchronises the device, then returns per class the launches recorded since
+ * the last collect, their summed duration (ms) and summed work. */
+int fmoe_profile_collect(int64_t *launches, double *milliseconds, double *work,
+                         int n_classes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FMOE_HIP_H */

@@ -1,0 +1,128 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads and exports
+every symbol include/fmoe_hip.h declares, the Python API has the reference's
+names and signatures, and bad arguments raise instead of reaching a kernel."""
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+import fastermoe_amd
+from fastermoe_amd import _lib, fmoe_native, functions, fused_functions, gates, layers, transformer
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "fmoe_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmoe_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 15
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in fmoe_hip.h but not exported"
+    assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header disagree"
+    assert lib.fmoe_abi_version() == 1
+
+
+def test_workspace_queries_run_without_a_gpu():
+    lib = _lib.load()
+    assert lib.fmoe_routing_workspace_bytes(65536, 256) >= (32 * 256 + 512) * 4
+    assert lib.fmoe_index_add_workspace_bytes(100, 50) >= 600
+    assert lib.fmoe_routing_workspace_bytes(-1, 4) == 0
+
+
+def test_python_api_names_and_signatures():
+    assert {"FMoE", "FMoELinear", "FMoETransformerMLP", "DistributedGroupedDataParallel"} <= set(dir(fastermoe_amd))
+    for name in ("count_by_gate", "prepare_forward", "MOEScatter", "MOELinear", "MOEGather", "MOECache",
+                 "ensure_comm", "AllGather", "Slice", "_local_scatter", "_local_gather"):
+        assert hasattr(functions, name)
+    assert hasattr(fused_functions, "MOEForward")
+    for name in ("NaiveGate", "GShardGate", "SwitchGate", "ZeroGate", "NoisyGate"):
+        assert hasattr(gates, name)
+    for name in ("expert_count", "assign_pos", "linear_forward", "linear_backward", "limit_by_capacity",
+                 "prune_gate_by_capacity", "fused_forward", "fused_backward"):
+        assert hasattr(fmoe_native, name)
+    # constructor signatures of fmoe/layers.py:169-184 and fmoe/transformer.py:96-112
+    p = inspect.signature(layers.FMoE.__init__).parameters
+    assert list(p)[1:] == ["num_expert", "d_model", "world_size", "mp_group", "moe_group", "top_k", "gate",
+                           "expert", "gate_hook", "policy_fn", "mask", "mask_dict", "enable_fuse"]
+    assert p["num_expert"].default == 32 and p["top_k"].default == 2 and p["d_model"].default == 1024
+    p = inspect.signature(transformer.FMoETransformerMLP.__init__).parameters
+    assert list(p)[1:] == ["num_expert", "d_model", "d_hidden", "world_size", "mp_group", "moe_group",
+                           "activation", "gate", "top_k", "expert_dp_comm", "gate_hook", "bias", "mask",
+                           "mask_dict"]
+    assert p["d_hidden"].default == 4096 and p["bias"].default is True
+    p = inspect.signature(functions.count_by_gate).parameters
+    assert list(p) == ["gate", "num_expert", "world_size", "require_pos"]
+
+
+def test_module_structure_and_parameter_names():
+    m = fastermoe_amd.FMoETransformerMLP(num_expert=4, d_model=16, d_hidden=32, top_k=2)
+    names = set(dict(m.named_parameters()))
+    assert names == {"gate.gate.weight", "gate.gate.bias", "experts.htoh4.weight", "experts.htoh4.bias",
+                     "experts.h4toh.weight", "experts.h4toh.bias"}
+    assert tuple(m.experts.htoh4.weight.shape) == (4, 32, 16)
+    assert tuple(m.experts.h4toh.weight.shape) == (4, 16, 32)
+    assert torch.count_nonzero(m.experts.htoh4.bias) == 0
+    # Kaiming-uniform over the 3-D tensor: bound 1/sqrt(out*in) (torch's fan_in for 3-D)
+    bound = (32 * 16) ** -0.5
+    assert m.experts.htoh4.weight.abs().max() <= bound
+    assert getattr(m.experts.htoh4.weight, "dp_comm") == "none"
+    assert getattr(m.gate.gate.weight, "dp_comm") == "moe"
+    nobias = fastermoe_amd.FMoETransformerMLP(num_expert=2, d_model=8, d_hidden=8, bias=False)
+    assert nobias.experts.htoh4.bias is None
+
+
+def test_multi_worker_is_refused():
+    with pytest.raises(NotImplementedError):
+        fastermoe_amd.FMoE(num_expert=2, d_model=8, world_size=2)
+    with pytest.raises(NotImplementedError):
+        functions.count_by_gate(torch.zeros(4, dtype=torch.int64), 2, 2)
+    with pytest.raises(NotImplementedError):
+        fastermoe_amd.DistributedGroupedDataParallel(torch.nn.Linear(2, 2))
+
+
+def test_cpu_tensors_are_rejected_not_computed():
+    g = torch.zeros(8, dtype=torch.int64)
+    with pytest.raises(ValueError, match="CUDA"):
+        fmoe_native.expert_count(g, torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(ValueError, match="CUDA"):
+        fmoe_native.linear_forward(torch.zeros(4, 8), torch.tensor([4]), torch.zeros(1, 8, 8), None)
+    with pytest.raises(ValueError, match="CUDA"):
+        fmoe_native.gather_rows(torch.zeros(4, 8), g)
+    with pytest.raises((ValueError, TypeError)):
+        fastermoe_amd.FMoETransformerMLP(num_expert=2, d_model=8, d_hidden=8)(torch.zeros(4, 8))
+
+
+def test_c_abi_rejects_bad_arguments_before_any_launch():
+    lib = _lib.load()
+    import ctypes
+    cnt = (ctypes.c_int64 * 2)(3, -1)
+    rc = lib.fmoe_linear_forward(None, None, None, None, ctypes.cast(cnt, ctypes.c_void_p), 2, 8, 8, _lib.BF16, None)
+    assert rc == -1 and b"negative" in lib.fmoe_last_error()
+    rc = lib.fmoe_linear_forward(None, None, None, None, ctypes.cast(cnt, ctypes.c_void_p), 2, 8, 8, 99, None)
+    assert rc == -1 and b"dtype" in lib.fmoe_last_error()
+    rc = lib.fmoe_expert_count(None, None, 10, 1 << 20, None)
+    assert rc == -2  # FMOE_ELIMIT
+    rc = lib.fmoe_assign_pos(None, None, None, 0, 10, 4, None, 0, None)
+    assert rc == -1
+    with pytest.raises(_lib.FmoeHipError):
+        _lib.check(rc)
+
+
+def test_activation_codes():
+    from fastermoe_amd.fused_functions import _activation_code
+    assert _activation_code(torch.nn.GELU()) == _lib.ACT_GELU
+    assert _activation_code(torch.nn.functional.gelu) == _lib.ACT_GELU
+    assert _activation_code(torch.nn.ReLU()) == _lib.ACT_RELU
+    assert _activation_code(torch.nn.Identity()) == _lib.ACT_NONE
+    with pytest.raises(NotImplementedError):
+        _activation_code(torch.nn.GELU(approximate="tanh"))
+    with pytest.raises(NotImplementedError):
+        _activation_code(torch.nn.Tanh())

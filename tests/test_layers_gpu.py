@@ -1,0 +1,275 @@
+"""GPU parity of the MoE modules against the brute-force oracle: the cases of the
+reference's tests/test_numerical.py (test_fmoe_linear, test_fmoe), tests/test_fused.py,
+tests/test_gates.py and tests/test_zero.py, plus the five benchmark configurations at
+reduced token counts."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import fastermoe_amd as fmoe
+from fastermoe_amd.gates import GShardGate, NaiveGate, SwitchGate, ZeroGate, NoisyGate
+from fastermoe_amd.layers import FMoE
+from fastermoe_amd.transformer import _Expert
+from oracle import moe as omoe
+from oracle import routing as orouting
+from helpers import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle(moe, x, idx, score, act, top_k):
+    e = moe.experts
+    return omoe.moe_mlp_forward_backward(
+        x, idx, score, e.htoh4.weight, e.htoh4.bias, e.h4toh.weight, e.h4toh.bias, act, top_k)
+
+
+def _compare(moe, x, act, top_k, dtype, grads_of_score=False):
+    x = x.clone().requires_grad_(True)
+    with torch.no_grad():
+        idx, score = moe.gate(x)
+    # fix the routing so that the layer and the oracle see the same gate output
+    moe.gate.forward = lambda inp: (idx, score)
+    moe.zero_grad()
+    out = moe(x)
+    out.mean().backward()
+    ref = _oracle(moe, x, idx, score, act, top_k)
+    tol = TOL[dtype]
+    e = moe.experts
+    got = {"out": out, "grad_inp": x.grad, "grad_w1": e.htoh4.weight.grad, "grad_w2": e.h4toh.weight.grad,
+           "grad_b1": e.htoh4.bias.grad if e.htoh4.bias is not None else None,
+           "grad_b2": e.h4toh.bias.grad if e.h4toh.bias is not None else None}
+    for name, val in got.items():
+        if val is None:
+            assert ref[name] is None
+            continue
+        assert rel_err(val, ref[name]) <= tol, (name, rel_err(val, ref[name]))
+    return got
+
+
+class MyMoE(FMoE):
+    """The reference tests' module (tests/test_numerical.py:65-81): FMoE with a fused
+    _Expert whose weights are N(0,1) from numpy's default_rng(1234)."""
+
+    def __init__(self, num_expert, d_model, d_hidden, top_k, activation, enable_fuse=False):
+        super().__init__(num_expert=num_expert, d_model=d_model, gate=NaiveGate, world_size=1, top_k=top_k,
+                         enable_fuse=enable_fuse)
+        self.experts = _Expert(num_expert, d_model, d_hidden, activation)
+        rng = np.random.default_rng(1234)
+        for lin in (self.experts.htoh4, self.experts.h4toh):
+            lin.weight.data = torch.from_numpy(rng.normal(0.0, 1.0, size=tuple(lin.weight.shape))).float()
+            lin.bias.data.zero_()
+
+
+@pytest.mark.parametrize("num_expert", [4, 8])
+@pytest.mark.parametrize("top_k", [2, 3])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+def test_fmoe_linear_reference_grid(num_expert, top_k, dtype, device):
+    """tests/test_numerical.py:84-207: batch 4, d_model 16, d_hidden 32, GELU, seed 42."""
+    torch.manual_seed(42)
+    moe = MyMoE(num_expert, 16, 32, top_k, torch.nn.functional.gelu).to(dtype).to(device)
+    x = torch.rand(4, 16).to(dtype).to(device)
+    got = _compare(moe, x, "gelu", top_k, dtype)
+    # the reference's own criterion: max abs error 1e-3 (5e-1 for half)
+    ref = _oracle(moe, x, *moe.gate(x), "gelu", top_k)
+    bound = 5e-1 if dtype in (torch.float16, torch.bfloat16) else 1e-3
+    assert (got["out"].double().cpu() - ref["out"]).abs().max() <= bound
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+@pytest.mark.parametrize("dtype,n,d,h,e,k,act", [
+    (torch.float32, 512, 512, 1024, 8, 2, "gelu"),      # config 1 shape
+    (torch.bfloat16, 1024, 1024, 4096, 16, 2, "gelu"),  # config 2 shape
+    (torch.bfloat16, 1024, 2048, 2048, 64, 1, "gelu"),  # config 3 shape (narrower hidden)
+    (torch.bfloat16, 1024, 4096, 3584, 8, 2, "gelu"),   # config 4 shape (quarter hidden)
+    (torch.bfloat16, 512, 2048, 1024, 256, 8, "gelu"),  # config 5 shape
+    (torch.float32, 200, 24, 40, 3, 2, "relu"),
+])
+def test_transformer_mlp_configs(fuse, dtype, n, d, h, e, k, act, device):
+    torch.manual_seed(42 + e)
+    activation = nn.GELU() if act == "gelu" else nn.ReLU()
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=activation)
+    moe.enable_fuse = fuse
+    # biases away from zero so that they matter
+    with torch.no_grad():
+        moe.experts.htoh4.bias.normal_(0, 0.02)
+        moe.experts.h4toh.bias.normal_(0, 0.02)
+    moe = moe.to(dtype).to(device)
+    x = torch.randn(n, d).to(dtype).to(device)
+    if e == 64:  # Zipf-skewed top-1 routing with empty experts and unit scores
+        p = torch.arange(1, e + 1, dtype=torch.float64) ** -1.2
+        idx = torch.multinomial(p / p.sum(), n, replacement=True).view(n, 1).to(device)
+        moe.gate.forward = lambda inp: (idx, torch.ones(n, 1, dtype=dtype, device=device))
+    _compare(moe, x, act, k, dtype)
+
+
+@pytest.mark.parametrize("chunks", ["1", "3", "7"])
+def test_fused_equals_unfused(chunks, device, monkeypatch):
+    """tests/test_fused.py:9-34 (forward, input grad, both weight grads within 1e-3),
+    for several chunk counts, with dropped slots and an expert left without tokens."""
+    monkeypatch.setenv("FMOE_FUSE_GRAN", chunks)
+    torch.manual_seed(0)
+    n, d, h, e, k = 300, 64, 96, 6, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU()).to(device)
+    with torch.no_grad():
+        moe.experts.htoh4.bias.normal_()
+        moe.experts.h4toh.bias.normal_()
+    x = torch.randn(n, d, device=device)
+    idx = torch.randint(0, e - 1, (n, k), device=device)      # expert e-1 gets nothing
+    idx[torch.rand(n, k, device=device) < 0.2] = -1
+    score = torch.rand(n, k, device=device)
+    moe.gate.forward = lambda inp: (idx, score)
+    results = []
+    for fuse in (False, True):
+        moe.enable_fuse = fuse
+        moe.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        out.mean().backward()
+        results.append([out, xi.grad] + [p.grad.clone() for p in moe.experts.parameters()])
+    for a, b in zip(*results):
+        assert (a - b).abs().max() <= 1e-3
+        assert rel_err(a, b) <= 1e-5
+    assert torch.count_nonzero(moe.experts.htoh4.weight.grad[e - 1]) == 0
+
+
+def test_reference_fused_entry_points(device):
+    """fmoe_native.fused_forward / fused_backward with the reference's argument lists
+    (fmoe/fused_functions.py:25-29,49-55): ReLU, no bias, one expert, d=4, h=8, 6 rows
+    (tests/test_fused.py:41-46)."""
+    from fastermoe_amd import fmoe_native
+    torch.manual_seed(1)
+    w1 = torch.randn(1, 8, 4, device=device, requires_grad=True)
+    w2 = torch.randn(1, 4, 8, device=device, requires_grad=True)
+    x = torch.randn(6, 4, device=device)
+    cnt = torch.tensor([6])
+    stored = torch.zeros(1, dtype=torch.bool)
+    out, gib, gmb, gob = fmoe_native.fused_forward(x, [[(w1, w2)]], cnt, cnt, stored, 6, 1, False)
+    ref = torch.relu(x @ w1[0].t()) @ w2[0].t()
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+    assert torch.equal(gib, x) and torch.allclose(gmb, torch.relu(x @ w1[0].t()), rtol=1e-5, atol=1e-6)
+    go = torch.randn(6, 4, device=device)
+    (grad_in,) = fmoe_native.fused_backward(gib, [[(w1, w2)]], gmb, gob, go, cnt, cnt, x, stored, 6, 6, 1, False)
+    xr = x.clone().requires_grad_(True)
+    w1r, w2r = w1.detach().clone().requires_grad_(True), w2.detach().clone().requires_grad_(True)
+    (torch.relu(xr @ w1r[0].t()) @ w2r[0].t()).backward(go)
+    assert torch.allclose(grad_in, xr.grad, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(w1.grad, w1r.grad, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(w2.grad, w2r.grad, rtol=1e-5, atol=1e-6)
+
+
+class _LinearExpert(nn.Module):
+    def __init__(self, d_model):
+        super().__init__()
+        self.model = nn.Sequential(nn.Linear(d_model, d_model * 2), nn.ReLU(), nn.Linear(d_model * 2, d_model))
+
+    def forward(self, x):
+        return self.model(x)
+
+
+@pytest.mark.parametrize("as_list", [False, True])
+def test_fmoe_generic_experts(as_list, device):
+    """tests/test_numerical.py:210-308,387-485: FMoE(expert=cls or list) against calling the
+    expert module of each slot one row at a time (tests/moe.py:52-75)."""
+    torch.manual_seed(42)
+    n, d, e, k = 12, 16, 4, 2
+    moe = FMoE(num_expert=e, d_model=d, top_k=k, gate=NaiveGate,
+               expert=[_LinearExpert] * e if as_list else _LinearExpert).to(device)
+    x = torch.rand(n, d, device=device, requires_grad=True)
+    idx, score = moe.gate(x)
+    out = moe(x)
+    rows = x.detach().repeat_interleave(k, dim=0)
+    per_slot = torch.stack([moe.experts[int(g)](rows[i]) for i, g in enumerate(idx.view(-1))])
+    ref = torch.bmm(score.view(n, 1, k), per_slot.view(n, k, d)).reshape(n, d)
+    assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
+    out.mean().backward()
+    assert x.grad is not None and all(p.grad is not None for p in moe.experts.parameters())
+
+
+@pytest.mark.parametrize("cap", [0.1, 1.1])
+@pytest.mark.parametrize("n,e", [(4096, 4), (1000, 16)])
+def test_gshard_gate(cap, n, e, device):
+    """tests/test_gates.py:25-64."""
+    torch.manual_seed(3)
+    gate = GShardGate(64, e, 1, capacity=(cap, cap)).to(device)
+    x = torch.rand(n, 64, device=device)
+    idx, val = gate(x)
+    assert idx.shape == (n, 2) and val.shape == (n, 2)
+    limit = math.ceil(cap * n)
+    counts = torch.bincount(idx[idx >= 0].view(-1), minlength=e)
+    assert int(counts.max()) <= limit
+    logits = gate.gate(x)
+    kept = idx >= 0
+    assert torch.equal(torch.gather(logits, 1, idx.clamp(min=0))[kept], val[kept])
+    assert gate.get_loss() is not None
+    # first-come-first-kept: what survives the capacity step is the oracle's pruning
+    top_val, top_idx = torch.topk(logits, 2, dim=-1, sorted=False)
+    _, _, pruned = orouting.limit_and_prune(top_idx.cpu().numpy(), e, limit)
+    survivors = torch.from_numpy(pruned).to(device)
+    assert bool(((idx == survivors) | (idx == -1)).all())
+    assert torch.equal(idx[:, 0], survivors[:, 0])      # random routing only touches column 1
+
+
+@pytest.mark.parametrize("cap", [0.1, 0.8])
+def test_switch_gate(cap, device):
+    """tests/test_gates.py:67-115."""
+    torch.manual_seed(4)
+    n, e = 2048, 8
+    gate = SwitchGate(32, e, 1, capacity=(cap, cap)).to(device)
+    gate.eval()
+    x = torch.rand(n, 32, device=device)
+    idx, score = gate(x)
+    assert idx.shape == (n, 1)
+    counts = torch.bincount(idx[idx >= 0].view(-1), minlength=e)
+    assert int(counts.max()) <= math.ceil(cap * n)
+    prob = torch.softmax(gate.gate(x).float(), dim=-1)
+    kept = (idx >= 0).view(-1)
+    assert torch.allclose(torch.gather(prob, 1, idx.clamp(min=0)).view(-1)[kept], score.view(-1)[kept])
+    assert torch.isfinite(gate.get_loss())
+
+
+def test_capacity_gate_in_layer(device):
+    """A GShard-gated layer end to end: dropped slots contribute zero rows."""
+    torch.manual_seed(5)
+    n, d, h, e = 512, 64, 128, 4
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=2,
+                                  gate=lambda *a: GShardGate(*a, capacity=(0.3, 0.3))).to(device)
+    x = torch.randn(n, d, device=device)
+    _compare(moe, x, "gelu", 2, torch.float32)
+
+
+def test_zero_and_noisy_gate_and_mask(device):
+    """tests/test_zero.py (runs without crashing, everything to expert 0) and the mask path."""
+    torch.manual_seed(6)
+    moe = fmoe.FMoETransformerMLP(num_expert=2, d_model=16, d_hidden=32, top_k=1, gate=ZeroGate).to(device)
+    x = torch.rand(10, 16, device=device)
+    y = moe(x)
+    e = moe.experts
+    ref = nn.functional.gelu(x @ e.htoh4.weight[0].t() + e.htoh4.bias[0]) @ e.h4toh.weight[0].t() + e.h4toh.bias[0]
+    assert torch.allclose(y, ref, rtol=1e-5, atol=1e-6)
+    # NoisyGate hands back flattened indices and [N,1,k] scores (fmoe/gates/noisy_gate.py:139-142)
+    noisy = NoisyGate(16, 4, 1, top_k=2).to(device)
+    nidx, nscore = noisy(torch.rand(10, 16, device=device))
+    assert nidx.shape == (20,) and nscore.shape == (10, 1, 2)
+    assert torch.allclose(nscore.sum(-1), torch.ones(10, 1, device=device)) and torch.isfinite(noisy.get_loss())
+    mask = torch.tensor([0, 1, 0, 0, 1, 0, 0, 0, 0, 0], device=device)
+    fill = torch.full((1, 16), 7.0, device=device)
+    masked = fmoe.FMoETransformerMLP(num_expert=2, d_model=16, d_hidden=32, top_k=1, mask=mask,
+                                     mask_dict={1: fill}).to(device)
+    ym = masked(x)
+    score = masked.gate(x)[1]
+    assert torch.allclose(ym[mask == 1], 7.0 * score[mask == 1].expand(-1, 16))
+
+
+def test_gate_hook_and_state_dict(device):
+    seen = {}
+    moe = fmoe.FMoETransformerMLP(num_expert=2, d_model=8, d_hidden=16, top_k=2,
+                                  gate_hook=lambda i, s, _: seen.update(idx=i, score=s)).to(device)
+    moe(torch.rand(5, 8, device=device))
+    assert seen["idx"].shape == (5, 2)
+    clone = fmoe.FMoETransformerMLP(num_expert=2, d_model=8, d_hidden=16, top_k=2).to(device)
+    clone.load_state_dict(moe.state_dict())
+    x = torch.rand(5, 8, device=device)
+    assert torch.equal(moe(x), clone(x))

@@ -1,0 +1,128 @@
+"""GPU parity of the per-expert linear (grouped GEMM) against the float64 oracle.
+
+Tolerances (relative to the largest reference magnitude): 1e-5 for float32,
+2e-2 for bfloat16 / float16, 1e-10 for float64."""
+import pytest
+import torch
+
+from fastermoe_amd import fmoe_native
+from fastermoe_amd.functions import MOELinear
+from oracle import moe as omoe
+from helpers import TOL, ragged_counts, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _reference(x, counts, w, b, gy):
+    x64 = x.double().requires_grad_(True)
+    w64 = w.double().requires_grad_(True)
+    b64 = b.double().requires_grad_(True) if b is not None else None
+    y = omoe.per_expert_linear(x64, counts, w64, b64)
+    y.backward(gy.double())
+    return y.detach(), x64.grad, w64.grad, (b64.grad if b is not None else None)
+
+
+CASES = [  # rows, experts, in, out, bias, empties
+    (1000, 4, 64, 128, True, 1),     # ragged segments, one empty expert
+    (777, 8, 256, 72, True, 2),      # out not a multiple of the tile, rows odd
+    (2048, 2, 512, 512, False, 0),   # full tiles
+    (300, 16, 40, 24, True, 5),      # many empty experts, tiny segments
+    (5, 3, 8, 8, True, 1),           # fewer rows than a tile
+    (0, 3, 16, 16, True, 3),         # no rows at all
+    (64, 2, 12, 20, True, 0),        # feature sizes off the vector grid -> any-shape kernel
+    (33, 1, 4, 8, False, 0),         # the shape of the reference's fused test (d=4, h=8)
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
+@pytest.mark.parametrize("rows,e,fin,fout,bias,empties", CASES)
+def test_linear_forward_backward(dtype, rows, e, fin, fout, bias, empties, device):
+    g = torch.Generator().manual_seed(rows + e + fin)
+    counts = ragged_counts(rows, e, g, empties) if rows else torch.zeros(e, dtype=torch.int64)
+    x = (torch.randn(rows, fin, generator=g)).to(dtype)
+    w = (torch.randn(e, fout, fin, generator=g) / fin ** 0.5).to(dtype)
+    b = torch.randn(e, fout, generator=g).to(dtype) if bias else None
+    gy = torch.randn(rows, fout, generator=g).to(dtype)
+    ref_y, ref_gx, ref_gw, ref_gb = _reference(x, counts, w, b, gy)
+
+    xd, wd, gyd = x.to(device), w.to(device), gy.to(device)
+    bd = b.to(device) if bias else None
+    y = fmoe_native.linear_forward(xd, counts, wd, bd)
+    tol = TOL[dtype]
+    assert y.shape == (rows, fout) and y.dtype == dtype
+    assert rel_err(y, ref_y) <= tol
+    gx, gw, gb = fmoe_native.linear_backward(gyd, xd, counts, wd, bd)
+    assert rel_err(gx, ref_gx) <= tol
+    assert rel_err(gw, ref_gw) <= tol
+    for ex in range(e):
+        if counts[ex] == 0:
+            assert torch.count_nonzero(gw[ex]) == 0      # cuda/parallel_linear.cuh:113-118
+    if bias:
+        assert rel_err(gb, ref_gb) <= tol
+    else:
+        assert gb is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_moelinear_autograd(dtype, device):
+    g = torch.Generator().manual_seed(1)
+    counts = torch.tensor([100, 0, 156, 44])
+    x = torch.randn(300, 96, generator=g).to(dtype)
+    w = (torch.randn(4, 160, 96, generator=g) / 10).to(dtype)
+    b = torch.randn(4, 160, generator=g).to(dtype)
+    gy = torch.randn(300, 160, generator=g).to(dtype)
+    ref_y, ref_gx, ref_gw, ref_gb = _reference(x, counts, w, b, gy)
+    xd = x.to(device).requires_grad_(True)
+    wd = w.to(device).requires_grad_(True)
+    bd = b.to(device).requires_grad_(True)
+    y = MOELinear.apply(xd, counts, wd, bd)
+    y.backward(gy.to(device))
+    tol = TOL[dtype]
+    assert rel_err(y, ref_y) <= tol and rel_err(xd.grad, ref_gx) <= tol
+    assert rel_err(wd.grad, ref_gw) <= tol and rel_err(bd.grad, ref_gb) <= tol
+
+
+def test_many_experts_split_into_several_launches(device):
+    """More experts than one launch's segment table holds (256)."""
+    g = torch.Generator().manual_seed(2)
+    e, fin, fout = 600, 32, 48
+    counts = torch.randint(0, 9, (e,), generator=g)
+    rows = int(counts.sum())
+    x = torch.randn(rows, fin, generator=g).bfloat16()
+    w = (torch.randn(e, fout, fin, generator=g) / 6).bfloat16()
+    gy = torch.randn(rows, fout, generator=g).bfloat16()
+    ref_y, ref_gx, ref_gw, _ = _reference(x, counts, w, None, gy)
+    y = fmoe_native.linear_forward(x.to(device), counts, w.to(device), None)
+    gx, gw, gb = fmoe_native.linear_backward(gy.to(device), x.to(device), counts, w.to(device), None)
+    assert rel_err(y, ref_y) <= 2e-2 and rel_err(gx, ref_gx) <= 2e-2 and rel_err(gw, ref_gw) <= 2e-2
+
+
+def test_linearity_at_full_width(device):
+    """config-4 feature sizes on a slice of its rows: f(a*x) = a*f(x) for a power of two
+    (exact in bf16), and zero input rows give exactly the bias."""
+    g = torch.Generator().manual_seed(3)
+    e, d, h = 2, 4096, 14336
+    counts = torch.tensor([700, 324])
+    x = torch.randn(1024, d, generator=g).bfloat16().to(device)
+    w = ((torch.rand(e, h, d, generator=g) * 2 - 1) * (d * h) ** -0.5).bfloat16().to(device)
+    b = torch.randn(e, h, generator=g).bfloat16().to(device)
+    y1 = fmoe_native.linear_forward(x, counts, w, None)
+    y4 = fmoe_native.linear_forward(x * 4, counts, w, None)
+    assert torch.equal(y4, y1 * 4)
+    yb = fmoe_native.linear_forward(torch.zeros_like(x), counts, w, b)
+    assert torch.equal(yb[:700], b[0].expand(700, h)) and torch.equal(yb[700:], b[1].expand(324, h))
+    ref = (x[:700].double().cpu() @ w[0].double().cpu().t())
+    assert rel_err(y1[:700], ref) <= 2e-2
+
+
+def test_validation_errors(device):
+    x = torch.zeros(4, 8, device=device)
+    w = torch.zeros(2, 8, 8, device=device)
+    with pytest.raises(ValueError, match="CPU"):
+        fmoe_native.linear_forward(x, torch.tensor([2, 2], device=device), w, None)
+    with pytest.raises(ValueError, match="sums to"):
+        fmoe_native.linear_forward(x, torch.tensor([2, 3]), w, None)
+    with pytest.raises(TypeError):
+        fmoe_native.linear_forward(x, torch.tensor([2, 2]), w.half(), None)
+    with pytest.raises(ValueError, match="features"):
+        fmoe_native.linear_forward(torch.zeros(4, 6, device=device), torch.tensor([2, 2]), w, None)
