@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libfmoe_hip.so")
+# FMOE_HIP_LIB points at another build of the same library (e.g. an experiment)
+LIB_PATH = os.environ.get("FMOE_HIP_LIB") or os.path.join(_HERE, "lib", "libfmoe_hip.so")
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64

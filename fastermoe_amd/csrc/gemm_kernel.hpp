@@ -17,7 +17,16 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 256;
+// Waves of a workgroup along C's rows and columns.  4 x 2 (512 threads, two waves per
+// SIMD, 64 x 128 per wave) keeps the matrix pipe fed while one wave sits at the
+// barrier or waits for LDS; 2 x 2 (256 threads, 128 x 128 per wave) halves the LDS
+// reads per MFMA.  FMOE_GEMM_WAVES_M selects at build time.
+#ifndef FMOE_GEMM_WAVES_M
+#define FMOE_GEMM_WAVES_M 4
+#endif
+constexpr int kWavesM = FMOE_GEMM_WAVES_M, kWavesN = 2;
+constexpr int kThreads = 64 * kWavesM * kWavesN;
+constexpr int kRowsPerPass = kThreads / 8;  // KC slabs: rows covered by one 16-byte load of every thread
 constexpr int kSlabBytes = 128;  // contraction bytes per row per slab
 constexpr int kStepsPerSlab = 4; // 32-byte contraction steps (two 16-byte chunks) per slab
 constexpr int kGroupM = 8;       // row tiles that share a column tile consecutively
@@ -101,7 +110,7 @@ template <typename T, int BM, int BN, int PSHAPE, int QSHAPE, int RAGGED, int EP
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
     constexpr int CE = Elem<T>::kPerChunk;           // elements per 16-byte chunk
     constexpr int BKE = kSlabBytes / (int)sizeof(T); // elements per slab row
-    constexpr int WM = BM / 2, WN = BN / 2;          // wave tile
+    constexpr int WM = BM / kWavesM, WN = BN / kWavesN;  // wave tile
     constexpr int TI = WN / 32, TJ = WM / 32;        // MFMA blocks per wave (cols, rows)
     constexpr int NP = BN * 8 / kThreads;            // 16-byte chunks per thread per slab
     constexpr int NQ = BM * 8 / kThreads;
@@ -175,87 +184,95 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    const int wave_m0 = (wave >> 1) * WM, wave_n0 = (wave & 1) * WN;
+    const int wave_m0 = (wave / kWavesN) * WM, wave_n0 = (wave % kWavesN) * WN;
 
     // -- global -> register -> LDS staging ---------------------------------------
-    // KC: chunk q = it*256 + t covers row q/8, chunk q%8 of the slab.
+    // Loads go through buffer instructions: an offset at or beyond the resource's
+    // size returns zeros, so rows outside the tile and the contraction tail need no
+    // branch -- their offset is replaced by kOutOfRange.
+    // KC: chunk q = it*256 + t covers row q/8, 16-byte chunk q%8 of the slab.
     // MC: chunk q covers contraction row q / CPR, 16-byte column chunk q % CPR.
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+    constexpr int P_CPR = BN / CE, P_KPI = kThreads / P_CPR;  // MC: chunks per k row, k rows per pass
+    constexpr int Q_CPR = BM / CE, Q_KPI = kThreads / Q_CPR;
+    const int kc_r = t >> 3, kc_c = t & 7;
+
+    uint32_t p_voff[NP], q_voff[NQ];
+    int p_lds, q_lds;  // byte offset of this thread's first chunk inside a slab
+    if (PSHAPE == kKC) {
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+            p_voff[it] = (it * kRowsPerPass + kc_r < p_valid)
+                             ? (uint32_t)(((int64_t)(it * kRowsPerPass + kc_r) * prm.ldp + kc_c * CE) * sizeof(T))
+                             : kOutOfRange;
+        p_lds = kc_r * kSlabBytes + ((kc_c ^ swz(kc_r)) << 4);
+    } else {
+        const int kk = t / P_CPR, c = t % P_CPR;
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+            p_voff[it] = (c * CE < p_valid)
+                             ? (uint32_t)(((int64_t)(it * P_KPI + kk) * prm.ldp + c * CE) * sizeof(T))
+                             : kOutOfRange;
+        p_lds = (kk * P_CPR + (c ^ mc_swz<T>(kk))) * 16;
+    }
+    if (QSHAPE == kKC) {
+#pragma unroll
+        for (int it = 0; it < NQ; ++it)
+            q_voff[it] = (it * kRowsPerPass + kc_r < q_valid)
+                             ? (uint32_t)(((int64_t)(it * kRowsPerPass + kc_r) * prm.ldq + kc_c * CE) * sizeof(T))
+                             : kOutOfRange;
+        q_lds = kc_r * kSlabBytes + ((kc_c ^ swz(kc_r)) << 4);
+    } else {
+        const int kk = t / Q_CPR, c = t % Q_CPR;
+#pragma unroll
+        for (int it = 0; it < NQ; ++it)
+            q_voff[it] = (c * CE < q_valid)
+                             ? (uint32_t)(((int64_t)(it * Q_KPI + kk) * prm.ldq + c * CE) * sizeof(T))
+                             : kOutOfRange;
+        q_lds = (kk * Q_CPR + (c ^ mc_swz<T>(kk))) * 16;
+    }
+    // bytes per pass inside the LDS slab (it -> it + 1)
+    constexpr int P_PASS = (PSHAPE == kKC) ? kRowsPerPass * kSlabBytes : P_KPI * P_CPR * 16;
+    constexpr int Q_PASS = (QSHAPE == kKC) ? kRowsPerPass * kSlabBytes : Q_KPI * Q_CPR * 16;
+
     u32x4 pg[NP], qg[NQ];
 
-    auto load_slab = [&](int k0) {
-        if (PSHAPE == kKC) {
-            const int r_t = t >> 3, c_t = t & 7;
-            const bool kok = k0 + c_t * CE < K;
-            const T *src = Pb + (int64_t)r_t * prm.ldp + k0 + c_t * CE;
+    // KC: the resource starts at contraction index k0 of the tile's first row and the
+    // chunk is dropped when it lies past K.  MC: the resource starts at contraction row
+    // k0 and is exactly as long as the rows that remain, so rows past K read as zero.
+    auto issue_loads = [&](int k0) {
+        const int k_left = K - k0;  // <= 0 past the end: everything reads as zero
+        {
+            const T *origin = (PSHAPE == kKC) ? Pb + k0 : Pb + (int64_t)k0 * prm.ldp;
+            int64_t bytes = (PSHAPE == kKC) ? (int64_t)kOutOfRange : (int64_t)k_left * prm.ldp * (int64_t)sizeof(T);
+            bytes = bytes < 0 ? 0 : (bytes > (int64_t)kOutOfRange ? (int64_t)kOutOfRange : bytes);
+            const __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
+            // sign bit of (k_left - 1 - first k of the chunk): set exactly when the chunk starts past K
+            const uint32_t past = (PSHAPE == kKC) ? ((uint32_t)(k_left - 1 - kc_c * CE) & kOutOfRange) : 0u;
 #pragma unroll
-            for (int it = 0; it < NP; ++it) {
-                pg[it] = u32x4{0, 0, 0, 0};
-                if (kok && it * 32 + r_t < p_valid) pg[it] = *(const u32x4 *)(src + (int64_t)it * 32 * prm.ldp);
-            }
-        } else {
-            constexpr int CPR = BN / CE, KPI = kThreads / CPR;
-            const int kk_t = t / CPR, c_t = t % CPR;
-            const bool rok = c_t * CE < p_valid;
-            const T *src = Pb + (int64_t)(k0 + kk_t) * prm.ldp + c_t * CE;
-#pragma unroll
-            for (int it = 0; it < NP; ++it) {
-                pg[it] = u32x4{0, 0, 0, 0};
-                if (rok && k0 + kk_t + it * KPI < K) pg[it] = *(const u32x4 *)(src + (int64_t)it * KPI * prm.ldp);
-            }
+            for (int it = 0; it < NP; ++it) pg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, p_voff[it] | past, 0, 0);
         }
-        if (QSHAPE == kKC) {
-            const int r_t = t >> 3, c_t = t & 7;
-            const bool kok = k0 + c_t * CE < K;
-            const T *src = Qb + (int64_t)r_t * prm.ldq + k0 + c_t * CE;
+        {
+            const T *origin = (QSHAPE == kKC) ? Qb + k0 : Qb + (int64_t)k0 * prm.ldq;
+            int64_t bytes = (QSHAPE == kKC) ? (int64_t)kOutOfRange : (int64_t)k_left * prm.ldq * (int64_t)sizeof(T);
+            bytes = bytes < 0 ? 0 : (bytes > (int64_t)kOutOfRange ? (int64_t)kOutOfRange : bytes);
+            const __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
+            const uint32_t past = (QSHAPE == kKC) ? ((uint32_t)(k_left - 1 - kc_c * CE) & kOutOfRange) : 0u;
 #pragma unroll
-            for (int it = 0; it < NQ; ++it) {
-                qg[it] = u32x4{0, 0, 0, 0};
-                if (kok && it * 32 + r_t < q_valid) qg[it] = *(const u32x4 *)(src + (int64_t)it * 32 * prm.ldq);
-            }
-        } else {
-            constexpr int CPR = BM / CE, KPI = kThreads / CPR;
-            const int kk_t = t / CPR, c_t = t % CPR;
-            const bool rok = c_t * CE < q_valid;
-            const T *src = Qb + (int64_t)(k0 + kk_t) * prm.ldq + c_t * CE;
-#pragma unroll
-            for (int it = 0; it < NQ; ++it) {
-                qg[it] = u32x4{0, 0, 0, 0};
-                if (rok && k0 + kk_t + it * KPI < K) qg[it] = *(const u32x4 *)(src + (int64_t)it * KPI * prm.ldq);
-            }
+            for (int it = 0; it < NQ; ++it) qg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, q_voff[it] | past, 0, 0);
         }
     };
 
-    auto store_slab = [&](int stage) {
-        unsigned char *sp = smem + stage * STAGE_BYTES;
-        unsigned char *sq = sp + P_BYTES;
-        if (PSHAPE == kKC) {
-            const int r_t = t >> 3, c_t = t & 7;
-            const int off = r_t * kSlabBytes + ((c_t ^ swz(r_t)) << 4);
+    auto write_lds = [&](int stage) {
+        unsigned char *sp = smem + stage * STAGE_BYTES + p_lds;
+        unsigned char *sq = smem + stage * STAGE_BYTES + P_BYTES + q_lds;
 #pragma unroll
-            for (int it = 0; it < NP; ++it) *(u32x4 *)(sp + off + it * 32 * kSlabBytes) = pg[it];
-        } else {
-            constexpr int CPR = BN / CE, KPI = kThreads / CPR;
-            const int kk_t = t / CPR, c_t = t % CPR;
+        for (int it = 0; it < NP; ++it) *(u32x4 *)(sp + it * P_PASS) = pg[it];
 #pragma unroll
-            for (int it = 0; it < NP; ++it) {
-                const int kk = kk_t + it * KPI;
-                *(u32x4 *)(sp + (kk * CPR + (c_t ^ mc_swz<T>(kk))) * 16) = pg[it];
-            }
-        }
-        if (QSHAPE == kKC) {
-            const int r_t = t >> 3, c_t = t & 7;
-            const int off = r_t * kSlabBytes + ((c_t ^ swz(r_t)) << 4);
-#pragma unroll
-            for (int it = 0; it < NQ; ++it) *(u32x4 *)(sq + off + it * 32 * kSlabBytes) = qg[it];
-        } else {
-            constexpr int CPR = BM / CE, KPI = kThreads / CPR;
-            const int kk_t = t / CPR, c_t = t % CPR;
-#pragma unroll
-            for (int it = 0; it < NQ; ++it) {
-                const int kk = kk_t + it * KPI;
-                *(u32x4 *)(sq + (kk * CPR + (c_t ^ mc_swz<T>(kk))) * 16) = qg[it];
-            }
-        }
+        for (int it = 0; it < NQ; ++it) *(u32x4 *)(sq + it * Q_PASS) = qg[it];
     };
 
     // -- fragments ---------------------------------------------------------------
@@ -301,30 +318,94 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[x][y][r] = 0.f;
 
+    // Main loop, one basic block per slab, software-pipelined by hand:
+    //   steps 0..2 : MFMAs of step ks, with the LDS reads of step ks+1 between them
+    //   step 3a    : first half of the MFMAs; the slab prefetched one iteration ago is
+    //                written to the other LDS buffer
+    //   barrier
+    //   step 3b    : second half of the MFMAs; the global loads of the slab after next
+    //                are issued and step 0 of the next slab is read from the other buffer
+    // so a global load has a whole slab of MFMAs to complete and no LDS read is waited
+    // for at the top of an iteration.  Past the last slab the loads return zeros and the
+    // extra LDS write lands in the buffer nobody reads, which keeps the body branch-free.
+    constexpr int kReadsPerFrag = (sizeof(T) == 2) ? 1 : 1;
+    constexpr int kPReads = TI * ((PSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : kReadsPerFrag);
+    constexpr int kQReads = TJ * ((QSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : kReadsPerFrag);
+    constexpr int kReads = kPReads + kQReads;                   // LDS read instructions per step
+    constexpr int kMfma = TI * TJ * (sizeof(T) == 4 ? 4 : 1);   // MFMA instructions per step
+    constexpr int kMfmaPerRead = 1;  // reads go out early in the step, the remaining MFMAs follow
+
     const int n_slabs = (K + BKE - 1) / BKE;
-    if (n_slabs > 0) {
-        load_slab(0);
-        store_slab(0);
-    }
+    u32x4 pf[2][TI], qf[2][TJ];
+    auto read_step = [&](int buf, const unsigned char *sp, const unsigned char *sq, int ks) {
+#ifdef FMOE_DEBUG_SKIP_LDS_READ
+        if (sp != smem) return;
+#endif
+#pragma unroll
+        for (int x = 0; x < TI; ++x) pf[buf][x] = frag(sp, PSHAPE, BN, wave_n0 + x * 32, ks);
+#pragma unroll
+        for (int y = 0; y < TJ; ++y) qf[buf][y] = frag(sq, QSHAPE, BM, wave_m0 + y * 32, ks);
+    };
+
+    issue_loads(0);
+    write_lds(0);
     __syncthreads();
+    issue_loads(BKE);
+    read_step(0, smem, smem + P_BYTES, 0);
+    __builtin_amdgcn_sched_barrier(0);
+
     for (int s = 0; s < n_slabs; ++s) {
-        if (s + 1 < n_slabs) load_slab((s + 1) * BKE);
         const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
         const unsigned char *sq = sp + P_BYTES;
 #pragma unroll
-        for (int ks = 0; ks < kStepsPerSlab; ++ks) {
-            u32x4 pf[TI], qf[TJ];
-#pragma unroll
-            for (int x = 0; x < TI; ++x) pf[x] = frag(sp, PSHAPE, BN, wave_n0 + x * 32, ks);
-#pragma unroll
-            for (int y = 0; y < TJ; ++y) qf[y] = frag(sq, QSHAPE, BM, wave_m0 + y * 32, ks);
+        for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
+            read_step((ks + 1) & 1, sp, sq, ks + 1);
 #pragma unroll
             for (int x = 0; x < TI; ++x)
 #pragma unroll
-                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[x], qf[y]);
+                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
+#pragma unroll
+            for (int i = 0; i < kReads; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // one LDS read
+                __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRead, 0);  // then MFMAs
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (s + 1 < n_slabs) store_slab((s + 1) & 1);
+        constexpr int kLast = (kStepsPerSlab - 1) & 1;
+        // step 3a
+#pragma unroll
+        for (int x = 0; x < TI / 2; ++x)
+#pragma unroll
+            for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+#ifndef FMOE_DEBUG_SKIP_LDS_WRITE
+        write_lds((s + 1) & 1);
+#endif
+#pragma unroll
+        for (int i = 0; i < kMfma / 2; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x200, (NP + NQ) / (kMfma / 2), 0); // then LDS writes
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef FMOE_DEBUG_SKIP_BARRIER
         __syncthreads();
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+        // step 3b
+#ifndef FMOE_DEBUG_SKIP_GLOBAL
+        issue_loads((s + 2) * BKE);
+#endif
+        read_step(0, smem + ((s + 1) & 1) * STAGE_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES + P_BYTES, 0);
+#pragma unroll
+        for (int x = TI / 2; x < TI; ++x)
+#pragma unroll
+            for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+#pragma unroll
+        for (int i = 0; i < kMfma / 2; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x020, (NP + NQ) / (kMfma / 2), 0);  // global loads
+            __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma / 2 - 1) / (kMfma / 2), 0);  // LDS reads
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // -- epilogue ------------------------------------------------------------------
