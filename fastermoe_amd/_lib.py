@@ -44,13 +44,15 @@ SIGNATURES = {
                                       _vp, _vp, _vp, _vp, _vp, _int, _vp]),
     "fmoe_fused_mlp_backward": (_int, [ctypes.POINTER(MlpParams), _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
+    "fmoe_combine_forward": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "fmoe_combine_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_profile_enable": (_int, [_int]),
     "fmoe_profile_classes": (_int, []),
     "fmoe_profile_collect": (_int, [_vp, _vp, _vp, _int]),
 }
 
 PROFILE_CLASSES = ["gemm_fwd", "gemm_dgrad", "gemm_wgrad", "bias_grad", "gather_rows", "scatter_rows",
-                   "reduce_slots", "index_add"]
+                   "reduce_slots", "index_add", "combine"]
 
 F32, BF16, F16, F64 = 0, 1, 2, 3
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2

@@ -6,6 +6,7 @@
 #include "profile.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace fmoe {
 namespace gemm {
@@ -82,6 +83,7 @@ struct GemmParams {
     const void *Q;     // row operand (supplies C's rows)
     void *C;
     const void *bias;  // per expert [n_cols] or null
+    void *bias_grad;   // ragged-K only: per expert [n_rows] column sums of Q (the output gradient), or null
     void *aux;         // see Epilogue
     int64_t ldp, ldq, ldc;      // leading dimensions in elements
     int64_t p_expert_stride;    // elements between two experts' P (0: P is row-indexed like Q)
@@ -266,13 +268,43 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         }
     };
 
-    auto write_lds = [&](int stage) {
+    // Bias gradient (weight-gradient product only): the workgroups of the first column
+    // tile also add up the rows of the Q slabs they stage, i.e. the column sums of the
+    // output gradient over the expert's rows.  Every thread keeps the sums of the CE
+    // columns of its chunk; they are combined across threads after the main loop.
+    float bsum[CE];
+#pragma unroll
+    for (int j = 0; j < CE; ++j) bsum[j] = 0.f;
+    auto add_chunk = [&](const u32x4 &v) {
+        if (sizeof(T) == 4) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bsum[j] += __uint_as_float(v[j]);
+        } else if (std::is_same<T, __bf16>::value) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                bsum[2 * j] += __uint_as_float(v[j] << 16);
+                bsum[2 * j + 1] += __uint_as_float(v[j] & 0xffff0000u);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                bsum[2 * j] += (float)__builtin_bit_cast(_Float16, (uint16_t)(v[j] & 0xffffu));
+                bsum[2 * j + 1] += (float)__builtin_bit_cast(_Float16, (uint16_t)(v[j] >> 16));
+            }
+        }
+    };
+
+    auto write_lds = [&](int stage, auto with_bias) {
         unsigned char *sp = smem + stage * STAGE_BYTES + p_lds;
         unsigned char *sq = smem + stage * STAGE_BYTES + P_BYTES + q_lds;
 #pragma unroll
         for (int it = 0; it < NP; ++it) *(u32x4 *)(sp + it * P_PASS) = pg[it];
 #pragma unroll
         for (int it = 0; it < NQ; ++it) *(u32x4 *)(sq + it * Q_PASS) = qg[it];
+        if constexpr (decltype(with_bias)::value) {
+#pragma unroll
+            for (int it = 0; it < NQ; ++it) add_chunk(qg[it]);
+        }
     };
 
     // -- fragments ---------------------------------------------------------------
@@ -347,65 +379,96 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         for (int y = 0; y < TJ; ++y) qf[buf][y] = frag(sq, QSHAPE, BM, wave_m0 + y * 32, ks);
     };
 
-    issue_loads(0);
-    write_lds(0);
-    __syncthreads();
-    issue_loads(BKE);
-    read_step(0, smem, smem + P_BYTES, 0);
-    __builtin_amdgcn_sched_barrier(0);
+    auto main_loop = [&](auto with_bias) {
+        issue_loads(0);
+        write_lds(0, with_bias);
+        __syncthreads();
+        issue_loads(BKE);
+        read_step(0, smem, smem + P_BYTES, 0);
+        __builtin_amdgcn_sched_barrier(0);
 
-    for (int s = 0; s < n_slabs; ++s) {
-        const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
-        const unsigned char *sq = sp + P_BYTES;
-#pragma unroll
-        for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
-            read_step((ks + 1) & 1, sp, sq, ks + 1);
-#pragma unroll
-            for (int x = 0; x < TI; ++x)
-#pragma unroll
-                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
-#pragma unroll
-            for (int i = 0; i < kReads; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // one LDS read
-                __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRead, 0);  // then MFMAs
+        for (int s = 0; s < n_slabs; ++s) {
+            const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
+            const unsigned char *sq = sp + P_BYTES;
+    #pragma unroll
+            for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
+                read_step((ks + 1) & 1, sp, sq, ks + 1);
+    #pragma unroll
+                for (int x = 0; x < TI; ++x)
+    #pragma unroll
+                    for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
+    #pragma unroll
+                for (int i = 0; i < kReads; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // one LDS read
+                    __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRead, 0);  // then MFMAs
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            constexpr int kLast = (kStepsPerSlab - 1) & 1;
+            // step 3a
+    #pragma unroll
+            for (int x = 0; x < TI / 2; ++x)
+    #pragma unroll
+                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+    #ifndef FMOE_DEBUG_SKIP_LDS_WRITE
+            write_lds((s + 1) & 1, with_bias);
+    #endif
+    #pragma unroll
+            for (int i = 0; i < kMfma / 2; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x200, (NP + NQ) / (kMfma / 2), 0); // then LDS writes
+            }
+            __builtin_amdgcn_sched_barrier(0);
+    #ifndef FMOE_DEBUG_SKIP_BARRIER
+            __syncthreads();
+    #endif
+            __builtin_amdgcn_sched_barrier(0);
+            // step 3b
+    #ifndef FMOE_DEBUG_SKIP_GLOBAL
+            issue_loads((s + 2) * BKE);
+    #endif
+            read_step(0, smem + ((s + 1) & 1) * STAGE_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES + P_BYTES, 0);
+    #pragma unroll
+            for (int x = TI / 2; x < TI; ++x)
+    #pragma unroll
+                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+    #pragma unroll
+            for (int i = 0; i < kMfma / 2; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x020, (NP + NQ) / (kMfma / 2), 0);  // global loads
+                __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma / 2 - 1) / (kMfma / 2), 0);  // LDS reads
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        constexpr int kLast = (kStepsPerSlab - 1) & 1;
-        // step 3a
+    };
+    bool want_bias = false;
+    if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) want_bias = prm.bias_grad != nullptr && nt == 0;
+    if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
+        if (want_bias) main_loop(std::true_type{});
+        else main_loop(std::false_type{});
+    } else {
+        main_loop(std::false_type{});
+    }
+
+    if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
+        if (want_bias) {
+            // thread t holds columns (t % Q_CPR) * CE .. + CE - 1 of contraction rows t / Q_CPR (mod Q_KPI);
+            // the Q_KPI partial sums of a column are added in ascending order
+            float *red = (float *)smem;
+            __syncthreads();
+            const int grp = t / Q_CPR, c = t % Q_CPR;
 #pragma unroll
-        for (int x = 0; x < TI / 2; ++x)
+            for (int j = 0; j < CE; ++j) red[grp * BM + c * CE + j] = bsum[j];
+            __syncthreads();
+            if (t < BM && t < q_valid) {
+                float sum = 0.f;
 #pragma unroll
-            for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
-#ifndef FMOE_DEBUG_SKIP_LDS_WRITE
-        write_lds((s + 1) & 1);
-#endif
-#pragma unroll
-        for (int i = 0; i < kMfma / 2; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x200, (NP + NQ) / (kMfma / 2), 0); // then LDS writes
+                for (int g = 0; g < Q_KPI; ++g) sum += red[g * BM + t];
+                T *dst = (T *)prm.bias_grad + (int64_t)expert * prm.n_rows + mt * BM + t;
+                if (prm.accumulate_first && ei == 0) sum += (float)*dst;
+                *dst = (T)sum;
+            }
         }
-        __builtin_amdgcn_sched_barrier(0);
-#ifndef FMOE_DEBUG_SKIP_BARRIER
-        __syncthreads();
-#endif
-        __builtin_amdgcn_sched_barrier(0);
-        // step 3b
-#ifndef FMOE_DEBUG_SKIP_GLOBAL
-        issue_loads((s + 2) * BKE);
-#endif
-        read_step(0, smem + ((s + 1) & 1) * STAGE_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES + P_BYTES, 0);
-#pragma unroll
-        for (int x = TI / 2; x < TI; ++x)
-#pragma unroll
-            for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
-#pragma unroll
-        for (int i = 0; i < kMfma / 2; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x020, (NP + NQ) / (kMfma / 2), 0);  // global loads
-            __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma / 2 - 1) / (kMfma / 2), 0);  // LDS reads
-        }
-        __builtin_amdgcn_sched_barrier(0);
     }
 
     // -- epilogue ------------------------------------------------------------------

@@ -324,13 +324,16 @@ int grouped_linear_wgrad(const LinearWgradArgs &a, const int64_t *counts, int64_
         GemmParams prm{};
         fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, 256);
         prm.profile_class = kProfGemmWgrad; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
-        prm.P = a.x; prm.Q = a.gy; prm.C = a.gw;
+        prm.P = a.x; prm.Q = a.gy; prm.C = a.gw; prm.bias_grad = fast ? a.gb : nullptr;
         prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
         prm.c_expert_stride = a.in_feat * a.out_feat;
         prm.n_cols = (int)a.in_feat; prm.n_rows = (int)a.out_feat;
         prm.accumulate_first = (e0 == plan.first && plan.accumulate_first) ? 1 : 0;
         if (int rc = dispatch<kWgrad>(prm, a.dtype, kEpiStore, fast, stream)) return rc;
     }
+    // the MFMA kernel folds the bias gradient into its first column tiles; the any-shape path does not
+    if (a.gb && !fast)
+        return grouped_bias_grad(a.gy, a.gb, a.out_feat, a.dtype, counts, n_expert, row_lo, row_hi, last_chunk, stream);
     return FMOE_OK;
 }
 
@@ -385,11 +388,11 @@ extern "C" int fmoe_linear_backward(const void *grad_y, const void *x, const voi
         if (int rc = grouped_linear_dgrad(d, expert_count_host, n_expert, 0, total, st)) return rc;
     }
     if (grad_w) {
-        LinearWgradArgs g{grad_y, x, grad_w, in_feat, out_feat, dtype};
+        LinearWgradArgs g{grad_y, x, grad_w, grad_b, in_feat, out_feat, dtype};
         if (int rc = grouped_linear_wgrad(g, expert_count_host, n_expert, 0, total, true, st)) return rc;
-    }
-    if (grad_b)
+    } else if (grad_b) {
         if (int rc = grouped_bias_grad(grad_y, grad_b, out_feat, dtype, expert_count_host, n_expert, 0, total, true, st))
             return rc;
+    }
     return FMOE_OK;
 }

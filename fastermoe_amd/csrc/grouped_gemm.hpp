@@ -47,6 +47,7 @@ struct LinearWgradArgs {
     const void *gy;     // [rows, out]
     const void *x;      // [rows, in]
     void *gw;           // [E, out, in]
+    void *gb;           // [E, out] bias gradient (column sums of gy per expert) or null
     int64_t in_feat, out_feat;
     int dtype;
 };

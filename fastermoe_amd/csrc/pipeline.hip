@@ -203,24 +203,18 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
         const bool is_last = c == last;
         if (hi == lo && !is_last) continue;
         if (hi > lo) FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
-        // second linear: g_mid = (g_out . W2) * act'(pre);  gW2 (+)= g_out^T . mid;  gb2 (+)= colsum(g_out)
+        // second linear: g_mid = (g_out . W2) * act'(pre);  gW2 (+)= g_out^T . mid;  gb2 (+)= colsum(g_out) (inside the weight-gradient kernel)
         const bool has_act = p->activation != FMOE_ACT_NONE;
         LinearDgradArgs d2{g_out, p->w2, g_mid, has_act ? buf_pre : nullptr, h, d, dt,
                            has_act ? kEpiDAct : kEpiStore, p->activation};
         if (int rc = grouped_linear_dgrad(d2, expert_count_host, E, lo, hi, l->compute)) return rc;
-        LinearWgradArgs w2{g_out, buf_mid, grad_w2, h, d, dt};
+        LinearWgradArgs w2{g_out, buf_mid, grad_w2, grad_b2, h, d, dt};
         if (int rc = grouped_linear_wgrad(w2, expert_count_host, E, lo, hi, is_last, l->compute)) return rc;
-        if (grad_b2)
-            if (int rc = grouped_bias_grad(g_out, grad_b2, d, dt, expert_count_host, E, lo, hi, is_last, l->compute))
-                return rc;
-        // first linear: g_in = g_mid . W1;  gW1 (+)= g_mid^T . buf_in;  gb1 (+)= colsum(g_mid)
+        // first linear: g_in = g_mid . W1;  gW1 (+)= g_mid^T . buf_in;  gb1 (+)= colsum(g_mid) (likewise)
         LinearDgradArgs d1{g_mid, p->w1, g_in, nullptr, d, h, dt, kEpiStore, FMOE_ACT_NONE};
         if (int rc = grouped_linear_dgrad(d1, expert_count_host, E, lo, hi, l->compute)) return rc;
-        LinearWgradArgs w1{g_mid, buf_in, grad_w1, d, h, dt};
+        LinearWgradArgs w1{g_mid, buf_in, grad_w1, grad_b1, d, h, dt};
         if (int rc = grouped_linear_wgrad(w1, expert_count_host, E, lo, hi, is_last, l->compute)) return rc;
-        if (grad_b1)
-            if (int rc = grouped_bias_grad(g_mid, grad_b1, h, dt, expert_count_host, E, lo, hi, is_last, l->compute))
-                return rc;
     }
     if (int rc = join_lanes(l, caller)) return rc;
     // grad_inp[t] = sum of the token's k expert-row gradients (rows of different

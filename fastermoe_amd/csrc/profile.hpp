@@ -20,7 +20,8 @@ enum ProfileClass {
     kProfScatterRows = 5,
     kProfReduceSlots = 6,
     kProfIndexAdd = 7,
-    kProfClasses = 8
+    kProfCombine = 8,
+    kProfClasses = 9
 };
 
 bool profile_enabled();

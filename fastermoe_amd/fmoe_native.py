@@ -196,6 +196,36 @@ def index_add_rows(inp, index, n_out):
     return out
 
 
+# ---- score-weighted combine ---------------------------------------------------------
+
+def combine_forward(x, score, n_tokens, top_k):
+    """out[t] = sum_j score[t,j] * x[t*top_k+j]  (torch.bmm(score[N,1,k], x[N,k,d]))."""
+    dt = _rows("x", x)
+    _dev("score", score, x.dtype)
+    if x.shape[0] != n_tokens * top_k or score.numel() != n_tokens * top_k:
+        raise ValueError("x must have n_tokens*top_k rows and score n_tokens*top_k entries")
+    out = torch.empty(n_tokens, x.shape[1], dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        check(_lib.load().fmoe_combine_forward(_ptr(x), _ptr(score), _ptr(out), n_tokens, top_k, x.shape[1], dt,
+                                               _stream(x)))
+    return out
+
+
+def combine_backward(grad_out, x, score, n_tokens, top_k):
+    """Returns (grad_x [N*top_k, d], grad_score [N, top_k])."""
+    dt = _rows("x", x)
+    _dev("grad_out", grad_out, x.dtype)
+    _dev("score", score, x.dtype)
+    if tuple(grad_out.shape) != (n_tokens, x.shape[1]):
+        raise ValueError(f"grad_out must be [{n_tokens}, {x.shape[1]}]")
+    grad_x = torch.empty_like(x)
+    grad_score = torch.empty(n_tokens, top_k, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        check(_lib.load().fmoe_combine_backward(_ptr(grad_out), _ptr(x), _ptr(score), _ptr(grad_x), _ptr(grad_score),
+                                                n_tokens, top_k, x.shape[1], dt, _stream(x)))
+    return grad_x, grad_score
+
+
 # ---- per-expert linear ----------------------------------------------------------
 
 def _check_linear(input_buf, expert_count, weight, bias):

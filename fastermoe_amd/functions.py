@@ -167,6 +167,26 @@ class MOEGather(Function):
         return _local_scatter(grad_out, pos), None, None, None, None, None, None, None
 
 
+class MOECombine(Function):
+    r"""``torch.bmm(gate_score[N,1,k], x[N,k,d])`` of fmoe/layers.py:321-322 as one
+    streaming kernel (fp32 accumulation, one rounding) with its backward."""
+
+    @staticmethod
+    def forward(ctx, x, gate_score, n_tokens, top_k):
+        x = x.contiguous()
+        gate_score = gate_score.contiguous()
+        ctx.save_for_backward(x, gate_score)
+        ctx.moe_args = n_tokens, top_k, gate_score.shape
+        return fmoe_native.combine_forward(x, gate_score, n_tokens, top_k)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, gate_score = ctx.saved_tensors
+        n_tokens, top_k, score_shape = ctx.moe_args
+        grad_x, grad_score = fmoe_native.combine_backward(grad_out.contiguous(), x, gate_score, n_tokens, top_k)
+        return grad_x, grad_score.view(score_shape), None, None
+
+
 class AllGather(Function):
     r"""fmoe/functions.py:333-349 (model-parallel group); one worker only."""
 

@@ -6,7 +6,7 @@ import os
 import torch
 import torch.nn as nn
 
-from .functions import (AllGather, MOECache, MOEGather, MOELinear, MOEScatter, Slice,
+from .functions import (AllGather, MOECache, MOECombine, MOEGather, MOELinear, MOEScatter, Slice,
                         _prepare_forward_ex, ensure_comm)
 from .gates import NaiveGate
 
@@ -210,7 +210,11 @@ class FMoE(nn.Module):
             x = fwd.view(-1, self.top_k, self.d_model)
 
         gate_score = gate_score.view(x.shape[0], 1, self.top_k)
-        x = torch.bmm(gate_score, x).reshape(-1, self.d_model)
+        if x.is_cuda and gate_score.dtype == x.dtype and x.is_floating_point():
+            # the bmm of fmoe/layers.py:321-322 as a streaming kernel
+            x = MOECombine.apply(x.reshape(-1, self.d_model), gate_score, x.shape[0], self.top_k)
+        else:
+            x = torch.bmm(gate_score, x).reshape(-1, self.d_model)
 
         if self.mp_size > 1:
             x = AllGather.apply(x, self.mp_rank, self.mp_size, self.mp_group)

@@ -129,6 +129,22 @@ int fmoe_index_add_rows(const void *inp, const int64_t *index, void *out,
                         int dtype, void *workspace, int64_t workspace_bytes,
                         void *stream);
 
+/* ---- score-weighted combination of the top-k expert outputs ------------- */
+
+/* out[t,:] = sum_{j<top_k} score[t,j] * x[t*top_k+j,:], accumulated in fp32.
+ * x [n_tokens*top_k, row], score [n_tokens, top_k] (same dtype), out
+ * [n_tokens, row].  Replaces torch.bmm(gate_score, x), fmoe/layers.py:321-322. */
+int fmoe_combine_forward(const void *x, const void *score, void *out,
+                         int64_t n_tokens, int64_t top_k, int64_t row_elems,
+                         int dtype, void *stream);
+
+/* Its backward: grad_x[t*top_k+j,:] = score[t,j] * grad_out[t,:] and
+ * grad_score[t,j] = <grad_out[t,:], x[t*top_k+j,:]>. */
+int fmoe_combine_backward(const void *grad_out, const void *x, const void *score,
+                          void *grad_x, void *grad_score, int64_t n_tokens,
+                          int64_t top_k, int64_t row_elems, int dtype,
+                          void *stream);
+
 /* ---- per-expert linear (one grouped GEMM over ragged row segments) ------ */
 
 /* y[seg_e,:] = x[seg_e,:] . w[e]^T (+ bias[e]); seg_e are consecutive row
@@ -206,7 +222,7 @@ int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *grad_out,
 /* Kernel classes, in the order of the arrays fmoe_profile_collect fills:
  * 0 grouped GEMM forward, 1 grouped GEMM data-grad, 2 grouped GEMM weight-grad
  * (work = flop); 3 bias grad, 4 gather rows, 5 scatter rows, 6 reduce slots,
- * 7 index add (work = algorithmic bytes).  No counterpart in the reference
+ * 7 index add, 8 score combine (work = algorithmic bytes).  No counterpart in the reference
  * (its cuda/utils/timer.hh is commented out); used by bench.py to time each
  * kernel with HIP events on the stream it is launched on. */
 int fmoe_profile_enable(int on);

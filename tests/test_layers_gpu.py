@@ -81,10 +81,10 @@ def test_fmoe_linear_reference_grid(num_expert, top_k, dtype, device):
 @pytest.mark.parametrize("fuse", [False, True])
 @pytest.mark.parametrize("dtype,n,d,h,e,k,act", [
     (torch.float32, 512, 512, 1024, 8, 2, "gelu"),      # config 1 shape
-    (torch.bfloat16, 1024, 1024, 4096, 16, 2, "gelu"),  # config 2 shape
-    (torch.bfloat16, 1024, 2048, 2048, 64, 1, "gelu"),  # config 3 shape (narrower hidden)
-    (torch.bfloat16, 1024, 4096, 3584, 8, 2, "gelu"),   # config 4 shape (quarter hidden)
-    (torch.bfloat16, 512, 2048, 1024, 256, 8, "gelu"),  # config 5 shape
+    (torch.bfloat16, 512, 1024, 4096, 16, 2, "gelu"),   # config 2 shape
+    (torch.bfloat16, 768, 1024, 2048, 64, 1, "gelu"),   # config 3 routing (64 experts, Zipf top-1), half width
+    (torch.bfloat16, 384, 4096, 3584, 8, 2, "gelu"),    # config 4 shape (quarter hidden)
+    (torch.bfloat16, 256, 512, 256, 256, 8, "gelu"),    # config 5 routing (256 experts, top-8), quarter width
     (torch.float32, 200, 24, 40, 3, 2, "relu"),
 ])
 def test_transformer_mlp_configs(fuse, dtype, n, d, h, e, k, act, device):

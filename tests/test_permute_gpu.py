@@ -106,6 +106,29 @@ def test_autograd_functions_match_torch_index_ops(device):
     assert torch.equal(out, torch.zeros(n * k, d, device=device).index_copy_(0, pos, y.detach()))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,k,d", [(300, 2, 1024), (64, 8, 40), (17, 3, 7), (5, 1, 16)])
+def test_combine_matches_bmm(dtype, n, k, d, device):
+    """The score-weighted top-k combination and its backward against torch.bmm in float64."""
+    from fastermoe_amd.functions import MOECombine
+    g = torch.Generator().manual_seed(n * k + d)
+    x = torch.randn(n * k, d, generator=g).to(dtype)
+    score = torch.randn(n, 1, k, generator=g).to(dtype)
+    go = torch.randn(n, d, generator=g).to(dtype)
+    x64 = x.detach().clone().double().requires_grad_(True)
+    s64 = score.detach().clone().double().requires_grad_(True)
+    ref = torch.bmm(s64, x64.view(n, k, d)).reshape(n, d)
+    ref.backward(go.double())
+    xd = x.detach().to(device).requires_grad_(True)
+    sd = score.detach().to(device).requires_grad_(True)
+    out = MOECombine.apply(xd, sd, n, k)
+    out.backward(go.to(device))
+    tol = {torch.float32: 1e-5, torch.float64: 1e-12}.get(dtype, 2e-2)
+    for got, want in ((out, ref), (xd.grad, x64.grad), (sd.grad, s64.grad)):
+        assert got.shape == want.shape
+        assert (got.double().cpu() - want).abs().max() <= tol * max(1.0, want.abs().max().item())
+
+
 def test_full_size_round_trip(device):
     """config-4 sized rows: scatter then gather restores every kept slot, dropped slots are zero;
     linearity of the reduction."""
