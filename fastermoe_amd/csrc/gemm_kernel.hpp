@@ -64,16 +64,35 @@ template <> struct Elem<float> {
     }
 };
 
+// erf by Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7): a reciprocal, an exponential and
+// five multiply-adds instead of the library routine's branches.  The same exponential,
+// exp(-x^2/2), is the Gaussian of GELU's derivative.
+struct GeluTerms {
+    float cdf;  // Phi(x) = 0.5 (1 + erf(x / sqrt 2))
+    float pdf;  // phi(x) = exp(-x^2 / 2) / sqrt(2 pi)
+};
+__device__ __forceinline__ GeluTerms gelu_terms(float x) {
+    const float z = fabsf(x) * 0.70710678118654752440f;
+    const float t = __builtin_amdgcn_rcpf(1.f + 0.3275911f * z);
+    const float e = __expf(-z * z);
+    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+    const float erf_abs = 1.f - poly * e;
+    const float half_erf = 0.5f * (x < 0.f ? -erf_abs : erf_abs);
+    return GeluTerms{0.5f + half_erf, 0.39894228040143267794f * e};
+}
+
 __device__ __forceinline__ float apply_act(float x, int act) {
     if (act == FMOE_ACT_RELU) return x > 0.f ? x : 0.f;
-    if (act == FMOE_ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
+    if (act == FMOE_ACT_GELU) return x * gelu_terms(x).cdf;
     return x;
 }
 
 __device__ __forceinline__ float act_grad(float x, int act) {
     if (act == FMOE_ACT_RELU) return x > 0.f ? 1.f : 0.f;
-    if (act == FMOE_ACT_GELU)
-        return 0.5f * (1.f + erff(x * 0.70710678118654752440f)) + x * 0.39894228040143267794f * __expf(-0.5f * x * x);
+    if (act == FMOE_ACT_GELU) {
+        const GeluTerms g = gelu_terms(x);
+        return g.cdf + x * g.pdf;
+    }
     return 1.f;
 }
 
@@ -472,67 +491,128 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     }
 
     // -- epilogue ------------------------------------------------------------------
-    // acc[x][y][4*g + i] is C(row = wave_m0 + 32*y + l32, col = wave_n0 + 32*x + 8*g + 4*h + i).
+    // acc[x][y][4*g + i] is C(row = wave_m0 + 32*y + l32, col = wave_n0 + 32*x + 8*g + 4*h + i):
+    // a lane owns 4 consecutive columns of 32 different rows, which written straight to
+    // memory would touch 32 cache lines per store.  Instead every wave passes its sub-tile
+    // through a private LDS staging area of [WM rows][256 B + 16 B pad] and moves it
+    // between LDS and memory with 16-byte accesses that cover whole 256-byte row pieces
+    // (4 rows per wave instruction).  Tiles that are read in the epilogue (the saved
+    // pre-activation, or C itself when accumulating) come in through the same area.
+    if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
+        if (want_bias) __syncthreads();  // the bias reduction used the start of LDS
+    }
+    constexpr int kStgRow = 256 + 16;            // bytes; the pad spreads rows over the banks
+    constexpr int CPP = 256 / (int)sizeof(T);    // C columns per pass through the staging area
+    constexpr int XPP = CPP / 32;                // 32-column MFMA blocks per pass
+    constexpr int NPASS = WN / CPP;
+    unsigned char *stg = smem + wave * (WM * kStgRow);
     const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride + n0 : nullptr;
     T *aux = prm.aux ? (T *)prm.aux + aux_off : nullptr;
     const bool accumulate = (RAGGED == kRaggedK) && prm.accumulate_first && ei == 0;
+    const int io_r = lane >> 4, io_c = lane & 15;  // coalesced side: 4 rows x 16 chunks per instruction
+
+    auto lds_sync = [&]() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup"); __builtin_amdgcn_wave_barrier(); };
+
+    // memory -> staging (rows/columns outside the tile read as zero)
+    auto stage_in = [&](const T *src, int col_base) {
 #pragma unroll
-    for (int y = 0; y < TJ; ++y) {
-        const int row = wave_m0 + y * 32 + l32;
-        if (row >= q_valid) continue;
+        for (int i = 0; i < WM / 4; ++i) {
+            const int r = i * 4 + io_r;
+            u32x4 v = u32x4{0, 0, 0, 0};
+            if (wave_m0 + r < q_valid && col_base + io_c * CE < p_valid)
+                v = *(const u32x4 *)(src + (int64_t)(wave_m0 + r) * prm.ldc + col_base + io_c * CE);
+            *(u32x4 *)(stg + r * kStgRow + io_c * 16) = v;
+        }
+    };
+    // staging -> memory
+    auto stage_out = [&](T *dst, int col_base) {
 #pragma unroll
-        for (int x = 0; x < TI; ++x) {
+        for (int i = 0; i < WM / 4; ++i) {
+            const int r = i * 4 + io_r;
+            const u32x4 v = *(const u32x4 *)(stg + r * kStgRow + io_c * 16);
+            if (wave_m0 + r < q_valid && col_base + io_c * CE < p_valid)
+                *(u32x4 *)(dst + (int64_t)(wave_m0 + r) * prm.ldc + col_base + io_c * CE) = v;
+        }
+    };
+    // accumulator side: 4 consecutive columns of one row
+    auto put4 = [&](int row, int col_in_pass, const float (&v)[4]) {
+        alignas(16) T res[4];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int col = wave_n0 + x * 32 + g * 8 + h * 4;
-                if (col >= p_valid) continue;
-                float v[4];
+        for (int i = 0; i < 4; ++i) res[i] = (T)v[i];
+        unsigned char *p = stg + row * kStgRow + col_in_pass * (int)sizeof(T);
+        if (sizeof(T) == 2) *(u32x2 *)p = *(const u32x2 *)res;
+        else *(u32x4 *)p = *(const u32x4 *)res;
+    };
+    auto get4 = [&](int row, int col_in_pass, float (&v)[4]) {
+        alignas(16) T in[4];
+        const unsigned char *p = stg + row * kStgRow + col_in_pass * (int)sizeof(T);
+        if (sizeof(T) == 2) *(u32x2 *)in = *(const u32x2 *)p;
+        else *(u32x4 *)in = *(const u32x4 *)p;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = acc[x][y][4 * g + i];
-                T *dst = Cb + (int64_t)row * prm.ldc + col;
-                if (bias) {
+        for (int i = 0; i < 4; ++i) v[i] = (float)in[i];
+    };
+
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) v[i] += (float)bias[col + i];
-                }
-                if (EPI == kEpiBiasAct) {
-                    if (aux) {
-                        alignas(16) T pre[4];
+    for (int pass = 0; pass < NPASS; ++pass) {
+        const int col_base = wave_n0 + pass * CPP;
+        // kind 0: the result; kind 1 (bias+act with a pre-activation buffer): the pre-activation first
+        constexpr int kKinds = (EPI == kEpiBiasAct) ? 2 : 1;
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) pre[i] = (T)v[i];
-                        T *adst = aux + (int64_t)row * prm.ldc + col;
-                        if (sizeof(T) == 2) *(u32x2 *)adst = *(const u32x2 *)pre;
-                        else *(u32x4 *)adst = *(const u32x4 *)pre;
+        for (int kind = kKinds - 1; kind >= 0; --kind) {
+            if (EPI == kEpiBiasAct && kind == 1 && !aux) continue;
+            const bool reads_tile = (EPI == kEpiDAct) || accumulate;
+            if (reads_tile) {
+                stage_in(EPI == kEpiDAct ? (const T *)aux : (const T *)Cb, col_base);
+                lds_sync();
+            }
+#pragma unroll
+            for (int xx = 0; xx < XPP; ++xx) {
+                const int x = pass * XPP + xx;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int cip = xx * 32 + g * 8 + h * 4;  // column inside this pass
+                    float b4[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (bias && col_base + cip < p_valid) {
+                        alignas(16) T bv[4];
+                        if (sizeof(T) == 2) *(u32x2 *)bv = *(const u32x2 *)(bias + col_base + cip);
+                        else *(u32x4 *)bv = *(const u32x4 *)(bias + col_base + cip);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) b4[i] = (float)bv[i];
                     }
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) v[i] = apply_act(v[i], prm.activation);
-                } else if (EPI == kEpiDAct) {
-                    alignas(16) T pre[4];
-                    const T *asrc = aux + (int64_t)row * prm.ldc + col;
-                    if (sizeof(T) == 2) *(u32x2 *)pre = *(const u32x2 *)asrc;
-                    else *(u32x4 *)pre = *(const u32x4 *)asrc;
+                    for (int y = 0; y < TJ; ++y) {
+                        const int row = y * 32 + l32;
+                        float v[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) v[i] *= act_grad((float)pre[i], prm.activation);
+                        for (int i = 0; i < 4; ++i) v[i] = acc[x][y][4 * g + i] + b4[i];
+                        if (EPI == kEpiBiasAct && kind == 0) {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) v[i] = apply_act(v[i], prm.activation);
+                        }
+                        if (reads_tile) {
+                            float in[4];
+                            get4(row, cip, in);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                v[i] = (EPI == kEpiDAct) ? v[i] * act_grad(in[i], prm.activation) : v[i] + in[i];
+                        }
+                        put4(row, cip, v);
+                    }
                 }
-                if (accumulate) {
-                    alignas(16) T old[4];
-                    if (sizeof(T) == 2) *(u32x2 *)old = *(const u32x2 *)dst;
-                    else *(u32x4 *)old = *(const u32x4 *)dst;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) v[i] += (float)old[i];
-                }
-                alignas(16) T res[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) res[i] = (T)v[i];
-                if (sizeof(T) == 2) *(u32x2 *)dst = *(const u32x2 *)res;
-                else *(u32x4 *)dst = *(const u32x4 *)res;
             }
+            lds_sync();
+            stage_out((EPI == kEpiBiasAct && kind == 1) ? aux : Cb, col_base);
+            lds_sync();
         }
     }
 }
 
 template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI>
 int launch_tiles(GemmParams &prm, hipStream_t stream) {
-    constexpr int smem = 2 * (BM + BN) * kSlabBytes;
+    // two slab buffers, or the epilogue's staging area (one [rows][256 B + 16 B] block per wave)
+    constexpr int smem_loop = 2 * (BM + BN) * kSlabBytes;
+    constexpr int smem_epi = kWavesM * kWavesN * (BM / kWavesM) * (256 + 16);
+    constexpr int smem = smem_loop > smem_epi ? smem_loop : smem_epi;
     static bool configured = false;
     auto kern = grouped_gemm_kernel<T, BM, BN, PS, QS, RG, EPI>;
     if (!configured) {

@@ -19,6 +19,7 @@
 #include "grouped_gemm.hpp"
 #include "permute.hpp"
 
+#include <cstdlib>
 #include <mutex>
 #include <vector>
 
@@ -102,6 +103,25 @@ int check_common(const char *who, const fmoe_mlp_params *p, const int64_t *count
     return FMOE_OK;
 }
 
+// Chunk c covers the sorted rows [bounds[c], bounds[c+1]).  The split is even, except
+// that a boundary moves to the nearest expert boundary when one lies within a quarter
+// of a chunk: an expert that is not cut needs no partial row tile and its weight
+// gradient is produced by one chunk instead of being accumulated over two.
+void chunk_bounds(const int64_t *counts, int64_t n_expert, int64_t n_rows, int n_chunks, int64_t *bounds) {
+    bounds[0] = 0;
+    for (int c = 1; c < n_chunks; ++c) {
+        const int64_t target = n_rows * c / n_chunks;
+        int64_t best = -1, start = 0;
+        for (int64_t e = 0; e <= n_expert; ++e) {
+            if (best < 0 || llabs(start - target) < llabs(best - target)) best = start;
+            if (e < n_expert) start += counts[e];
+        }
+        int64_t b = (llabs(best - target) * 4 * n_chunks <= n_rows) ? best : target;
+        bounds[c] = b < bounds[c - 1] ? bounds[c - 1] : b;
+    }
+    bounds[n_chunks] = n_rows;
+}
+
 inline const char *at(const void *base, int64_t row, int64_t row_elems, int dtype) {
     return static_cast<const char *>(base) + row * row_elems * dtype_bytes(dtype);
 }
@@ -132,13 +152,15 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     DeviceLanes *l;
     if (int rc = get_lanes(&l)) return rc;
     if (int rc = fork_lanes(l, caller)) return rc;
+    int64_t bounds[kMaxChunks + 1];
+    chunk_bounds(expert_count_host, E, n_rows, n_chunks, bounds);
 
     // dropped slots become zero rows; independent of everything else
     if (n_rows < n_slots)
         if (int rc = permute_zero_unmapped(slot_to_row, out, n_slots, d, dt, l->out)) return rc;
 
     for (int c = 0; c < n_chunks; ++c) {
-        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         // permute-in: buf_in[r] = inp[pos[r] / top_k]
         if (int rc = permute_gather_rows(inp, pos + lo, top_k, at(buf_in, lo, d, dt), hi - lo, n_tokens, d, dt, l->in))
@@ -146,7 +168,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
         FMOE_HIP_CHECK(hipEventRecord(l->in_ready[c], l->in));
     }
     for (int c = 0; c < n_chunks; ++c) {
-        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
         LinearForwardArgs f1{buf_in, p->w1, p->b1, buf_mid, buf_pre, d, h, dt, kEpiBiasAct, p->activation};
@@ -156,7 +178,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
         FMOE_HIP_CHECK(hipEventRecord(l->out_ready[c], l->compute));
     }
     for (int c = 0; c < n_chunks; ++c) {
-        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         FMOE_HIP_CHECK(hipStreamWaitEvent(l->out, l->out_ready[c], 0));
         // permute-out: out[pos[r]] = buf_out[r]
@@ -187,9 +209,11 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     DeviceLanes *l;
     if (int rc = get_lanes(&l)) return rc;
     if (int rc = fork_lanes(l, caller)) return rc;
+    int64_t bounds[kMaxChunks + 1];
+    chunk_bounds(expert_count_host, E, n_rows, n_chunks, bounds);
 
     for (int c = 0; c < n_chunks; ++c) {
-        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         // permute-in: g_out[r] = grad_out[pos[r]]
         if (int rc = permute_gather_rows(grad_out, pos + lo, 1, at(g_out, lo, d, dt), hi - lo, n_slots, d, dt, l->in))
@@ -199,7 +223,7 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     // The last chunk (even when it is empty) also zero-fills the experts without rows.
     int last = n_chunks - 1;
     for (int c = 0; c < n_chunks; ++c) {
-        const int64_t lo = n_rows * c / n_chunks, hi = n_rows * (c + 1) / n_chunks;
+        const int64_t lo = bounds[c], hi = bounds[c + 1];
         const bool is_last = c == last;
         if (hi == lo && !is_last) continue;
         if (hi > lo) FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
