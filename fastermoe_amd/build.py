@@ -67,6 +67,9 @@ def build(jobs=None, verbose=False):
     objs = [os.path.join(OBJ, u[1]) for u in units]
     link = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB] + objs
     subprocess.check_call(link)
+    # a kernel the compiler dropped shows up as an undefined symbol when the library is loaded
+    import ctypes
+    ctypes.CDLL(LIB)
     return LIB
 
 

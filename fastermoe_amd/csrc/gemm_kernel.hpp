@@ -25,6 +25,10 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #ifndef FMOE_GEMM_WAVES_M
 #define FMOE_GEMM_WAVES_M 4
 #endif
+// 1: global loads write LDS directly (buffer_load ... lds); 0: through registers
+#ifndef FMOE_GEMM_LDS_DMA
+#define FMOE_GEMM_LDS_DMA 1
+#endif
 constexpr int kWavesM = FMOE_GEMM_WAVES_M, kWavesN = 2;
 constexpr int kThreads = 64 * kWavesM * kWavesN;
 constexpr int kRowsPerPass = kThreads / 8;  // KC slabs: rows covered by one 16-byte load of every thread
@@ -129,6 +133,7 @@ template <typename T> __device__ __forceinline__ int mc_swz(int k) { return size
 // ---- the kernel ---------------------------------------------------------------
 template <typename T, int BM, int BN, int PSHAPE, int QSHAPE, int RAGGED, int EPI>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
     constexpr int CE = Elem<T>::kPerChunk;           // elements per 16-byte chunk
     constexpr int BKE = kSlabBytes / (int)sizeof(T); // elements per slab row
     constexpr int WM = BM / kWavesM, WN = BN / kWavesN;  // wave tile
@@ -217,53 +222,89 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
     constexpr int P_CPR = BN / CE, P_KPI = kThreads / P_CPR;  // MC: chunks per k row, k rows per pass
     constexpr int Q_CPR = BM / CE, Q_KPI = kThreads / Q_CPR;
-    const int kc_r = t >> 3, kc_c = t & 7;
+    constexpr int kPassBytes = kThreads * 16;  // LDS bytes filled by one 16-byte load of every thread
 
+    // Slot q = it*kThreads + t of a slab is filled by thread t in pass it, so a wave fills
+    // 1 KiB of consecutive LDS per load.  The swizzle is applied on the memory side: the
+    // thread fetches the chunk that belongs in its slot.
+    //   KC: slot q is row q/8, position q%8, and holds chunk (q%8) ^ swz(row)
+    //   MC: slot q is contraction row q/CPR, position q%CPR, and holds chunk (q%CPR) ^ mc_swz(k)
     uint32_t p_voff[NP], q_voff[NQ];
-    int p_lds, q_lds;  // byte offset of this thread's first chunk inside a slab
+    int p_kc_chunk = 0, q_kc_chunk = 0;  // KC: logical chunk of this thread (same in every pass)
     if (PSHAPE == kKC) {
+        const int r = t >> 3;
+        p_kc_chunk = (t & 7) ^ swz(r);
 #pragma unroll
         for (int it = 0; it < NP; ++it)
-            p_voff[it] = (it * kRowsPerPass + kc_r < p_valid)
-                             ? (uint32_t)(((int64_t)(it * kRowsPerPass + kc_r) * prm.ldp + kc_c * CE) * sizeof(T))
+            p_voff[it] = (it * kRowsPerPass + r < p_valid)
+                             ? (uint32_t)(((int64_t)(it * kRowsPerPass + r) * prm.ldp + p_kc_chunk * CE) * sizeof(T))
                              : kOutOfRange;
-        p_lds = kc_r * kSlabBytes + ((kc_c ^ swz(kc_r)) << 4);
     } else {
-        const int kk = t / P_CPR, c = t % P_CPR;
+        const int kk = t / P_CPR, c = (t % P_CPR) ^ mc_swz<T>(kk);
 #pragma unroll
         for (int it = 0; it < NP; ++it)
             p_voff[it] = (c * CE < p_valid)
                              ? (uint32_t)(((int64_t)(it * P_KPI + kk) * prm.ldp + c * CE) * sizeof(T))
                              : kOutOfRange;
-        p_lds = (kk * P_CPR + (c ^ mc_swz<T>(kk))) * 16;
     }
     if (QSHAPE == kKC) {
+        const int r = t >> 3;
+        q_kc_chunk = (t & 7) ^ swz(r);
 #pragma unroll
         for (int it = 0; it < NQ; ++it)
-            q_voff[it] = (it * kRowsPerPass + kc_r < q_valid)
-                             ? (uint32_t)(((int64_t)(it * kRowsPerPass + kc_r) * prm.ldq + kc_c * CE) * sizeof(T))
+            q_voff[it] = (it * kRowsPerPass + r < q_valid)
+                             ? (uint32_t)(((int64_t)(it * kRowsPerPass + r) * prm.ldq + q_kc_chunk * CE) * sizeof(T))
                              : kOutOfRange;
-        q_lds = kc_r * kSlabBytes + ((kc_c ^ swz(kc_r)) << 4);
     } else {
-        const int kk = t / Q_CPR, c = t % Q_CPR;
+        const int kk = t / Q_CPR, c = (t % Q_CPR) ^ mc_swz<T>(kk);
 #pragma unroll
         for (int it = 0; it < NQ; ++it)
             q_voff[it] = (c * CE < q_valid)
                              ? (uint32_t)(((int64_t)(it * Q_KPI + kk) * prm.ldq + c * CE) * sizeof(T))
                              : kOutOfRange;
-        q_lds = (kk * Q_CPR + (c ^ mc_swz<T>(kk))) * 16;
     }
-    // bytes per pass inside the LDS slab (it -> it + 1)
-    constexpr int P_PASS = (PSHAPE == kKC) ? kRowsPerPass * kSlabBytes : P_KPI * P_CPR * 16;
-    constexpr int Q_PASS = (QSHAPE == kKC) ? kRowsPerPass * kSlabBytes : Q_KPI * Q_CPR * 16;
 
-    u32x4 pg[NP], qg[NQ];
+    // Direct-to-LDS loads pay off when both slabs are KC (forward); with an MC slab the
+    // register path measured faster, so the choice is per product.
+    constexpr bool kDma = FMOE_GEMM_LDS_DMA != 0;
+    // With an MC slab the fragments are read by ds_read_b64_tr_b16, and the compiler puts a
+    // full vmcnt(0) wait between a direct-to-LDS load and any such read that follows it
+    // (it cannot tell the two LDS buffers apart), which would serialise the pipeline.  For
+    // those products the load is emitted as inline assembly, which the compiler does not
+    // track; the one wait that is needed (before the barrier) is written out by hand.
+    constexpr bool kDmaAsm = kDma && (PSHAPE == kMC || QSHAPE == kMC);
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)smem;
+    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    auto dma_asm = [&](const T *origin, int64_t bytes, uint32_t lds_off, uint32_t voff) {
+        const uint64_t a = (uint64_t)origin;
+        i32x4 rs;
+        rs[0] = (int)(uint32_t)a;
+        rs[1] = (int)((uint32_t)(a >> 32) & 0xffffu);
+        rs[2] = (int)bytes;
+        rs[3] = kRsrcFlags;
+        rs[0] = __builtin_amdgcn_readfirstlane(rs[0]);
+        rs[1] = __builtin_amdgcn_readfirstlane(rs[1]);
+        rs[2] = __builtin_amdgcn_readfirstlane(rs[2]);
+        const uint32_t lds_addr = __builtin_amdgcn_readfirstlane(lds_base + lds_off);
+        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(rs)
+                     : "memory");
+    };
+    u32x4 pg[NP], qg[NQ];  // register path only
 
     // KC: the resource starts at contraction index k0 of the tile's first row and the
     // chunk is dropped when it lies past K.  MC: the resource starts at contraction row
     // k0 and is exactly as long as the rows that remain, so rows past K read as zero.
-    auto issue_loads = [&](int k0) {
+    // With FMOE_GEMM_LDS_DMA the loads write LDS directly (buffer_load ... lds: lane i of
+    // a wave lands at base + 16 i, out-of-range lanes land as zeros) into buffer `stage`;
+    // otherwise they return in registers and write_lds() stores them.
+    auto issue_loads = [&](int k0, int stage) {
         const int k_left = K - k0;  // <= 0 past the end: everything reads as zero
+        unsigned char *sp = smem + stage * STAGE_BYTES + wave * 1024;
+        unsigned char *sq = sp + P_BYTES;
+        (void)sp; (void)sq;
         {
             const T *origin = (PSHAPE == kKC) ? Pb + k0 : Pb + (int64_t)k0 * prm.ldp;
             int64_t bytes = (PSHAPE == kKC) ? (int64_t)kOutOfRange : (int64_t)k_left * prm.ldp * (int64_t)sizeof(T);
@@ -271,9 +312,17 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             const __amdgpu_buffer_rsrc_t rsrc =
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
             // sign bit of (k_left - 1 - first k of the chunk): set exactly when the chunk starts past K
-            const uint32_t past = (PSHAPE == kKC) ? ((uint32_t)(k_left - 1 - kc_c * CE) & kOutOfRange) : 0u;
+            const uint32_t past = (PSHAPE == kKC) ? ((uint32_t)(k_left - 1 - p_kc_chunk * CE) & kOutOfRange) : 0u;
 #pragma unroll
-            for (int it = 0; it < NP; ++it) pg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, p_voff[it] | past, 0, 0);
+            for (int it = 0; it < NP; ++it) {
+                if constexpr (kDmaAsm)
+                    dma_asm(origin, bytes, stage * STAGE_BYTES + wave_u * 1024 + it * kPassBytes, p_voff[it] | past);
+                else if constexpr (kDma)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(sp + it * kPassBytes),
+                                                             16, p_voff[it] | past, 0, 0, 0);
+                else
+                    pg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, p_voff[it] | past, 0, 0);
+            }
         }
         {
             const T *origin = (QSHAPE == kKC) ? Qb + k0 : Qb + (int64_t)k0 * prm.ldq;
@@ -281,9 +330,17 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             bytes = bytes < 0 ? 0 : (bytes > (int64_t)kOutOfRange ? (int64_t)kOutOfRange : bytes);
             const __amdgpu_buffer_rsrc_t rsrc =
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
-            const uint32_t past = (QSHAPE == kKC) ? ((uint32_t)(k_left - 1 - kc_c * CE) & kOutOfRange) : 0u;
+            const uint32_t past = (QSHAPE == kKC) ? ((uint32_t)(k_left - 1 - q_kc_chunk * CE) & kOutOfRange) : 0u;
 #pragma unroll
-            for (int it = 0; it < NQ; ++it) qg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, q_voff[it] | past, 0, 0);
+            for (int it = 0; it < NQ; ++it) {
+                if constexpr (kDmaAsm)
+                    dma_asm(origin, bytes, stage * STAGE_BYTES + P_BYTES + wave_u * 1024 + it * kPassBytes, q_voff[it] | past);
+                else if constexpr (kDma)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(sq + it * kPassBytes),
+                                                             16, q_voff[it] | past, 0, 0, 0);
+                else
+                    qg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, q_voff[it] | past, 0, 0);
+            }
         }
     };
 
@@ -313,16 +370,25 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         }
     };
 
+    // Registers -> LDS (register path), or nothing (the loads wrote LDS themselves); in
+    // both cases the bias-gradient workgroups add up the chunks this thread staged.
     auto write_lds = [&](int stage, auto with_bias) {
-        unsigned char *sp = smem + stage * STAGE_BYTES + p_lds;
-        unsigned char *sq = smem + stage * STAGE_BYTES + P_BYTES + q_lds;
+        unsigned char *sp = smem + stage * STAGE_BYTES + t * 16;
+        unsigned char *sq = sp + P_BYTES;
+        if constexpr (kDma) {
+            if constexpr (decltype(with_bias)::value) {
 #pragma unroll
-        for (int it = 0; it < NP; ++it) *(u32x4 *)(sp + it * P_PASS) = pg[it];
+                for (int it = 0; it < NQ; ++it) add_chunk(*(const u32x4 *)(sq + it * kPassBytes));
+            }
+        } else {
 #pragma unroll
-        for (int it = 0; it < NQ; ++it) *(u32x4 *)(sq + it * Q_PASS) = qg[it];
-        if constexpr (decltype(with_bias)::value) {
+            for (int it = 0; it < NP; ++it) *(u32x4 *)(sp + it * kPassBytes) = pg[it];
 #pragma unroll
-            for (int it = 0; it < NQ; ++it) add_chunk(qg[it]);
+            for (int it = 0; it < NQ; ++it) *(u32x4 *)(sq + it * kPassBytes) = qg[it];
+            if constexpr (decltype(with_bias)::value) {
+#pragma unroll
+                for (int it = 0; it < NQ; ++it) add_chunk(qg[it]);
+            }
         }
     };
 
@@ -389,9 +455,6 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     const int n_slabs = (K + BKE - 1) / BKE;
     u32x4 pf[2][TI], qf[2][TJ];
     auto read_step = [&](int buf, const unsigned char *sp, const unsigned char *sq, int ks) {
-#ifdef FMOE_DEBUG_SKIP_LDS_READ
-        if (sp != smem) return;
-#endif
 #pragma unroll
         for (int x = 0; x < TI; ++x) pf[buf][x] = frag(sp, PSHAPE, BN, wave_n0 + x * 32, ks);
 #pragma unroll
@@ -399,24 +462,87 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     };
 
     auto main_loop = [&](auto with_bias) {
-        issue_loads(0);
-        write_lds(0, with_bias);
+      if constexpr (kDma) {
+        // Direct-to-LDS pipeline.  Buffer A = s&1 is computed from, buffer B = the other
+        // one holds (or is receiving) slab s+1.  Per slab:
+        //   steps 0..2 : MFMAs of step ks, LDS reads of step ks+1 between them
+        //   step 3a    : first half of the last step's MFMAs, then wait for this wave's
+        //                loads of slab s+1
+        //   barrier    : slab s+1 is complete in B and nobody reads A any more
+        //   step 3b    : second half of the MFMAs; slab s+2 is requested into A and
+        //                step 0 of slab s+1 is read from B
+        constexpr int kVmcnt0 = 0x0F70;  // s_waitcnt vmcnt(0), other counters untouched
+        issue_loads(0, 0);
+        __builtin_amdgcn_s_waitcnt(kVmcnt0);
         __syncthreads();
-        issue_loads(BKE);
+        if constexpr (decltype(with_bias)::value) write_lds(0, with_bias);
+        issue_loads(BKE, 1);
         read_step(0, smem, smem + P_BYTES, 0);
         __builtin_amdgcn_sched_barrier(0);
 
         for (int s = 0; s < n_slabs; ++s) {
             const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
             const unsigned char *sq = sp + P_BYTES;
-    #pragma unroll
+#pragma unroll
             for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
                 read_step((ks + 1) & 1, sp, sq, ks + 1);
-    #pragma unroll
+#pragma unroll
                 for (int x = 0; x < TI; ++x)
-    #pragma unroll
+#pragma unroll
                     for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
-    #pragma unroll
+#pragma unroll
+                for (int i = 0; i < kReads; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRead, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            constexpr int kLast = (kStepsPerSlab - 1) & 1;
+#pragma unroll
+            for (int x = 0; x < TI / 2; ++x)
+#pragma unroll
+                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(kVmcnt0);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (decltype(with_bias)::value) write_lds((s + 1) & 1, with_bias);
+            issue_loads((s + 2) * BKE, s & 1);
+            read_step(0, smem + ((s + 1) & 1) * STAGE_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES + P_BYTES, 0);
+#pragma unroll
+            for (int x = TI / 2; x < TI; ++x)
+#pragma unroll
+                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+#pragma unroll
+            for (int i = 0; i < kMfma / 2; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma / 2 - 1) / (kMfma / 2), 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, (NP + NQ) / (kMfma / 2), 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the loads requested past the last slab (all out of range) must land before LDS is reused
+        __builtin_amdgcn_s_waitcnt(kVmcnt0);
+        __syncthreads();
+      } else {
+        issue_loads(0, 0);
+        write_lds(0, with_bias);
+        __syncthreads();
+        issue_loads(BKE, 0);
+        read_step(0, smem, smem + P_BYTES, 0);
+        __builtin_amdgcn_sched_barrier(0);
+
+        for (int s = 0; s < n_slabs; ++s) {
+            const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
+            const unsigned char *sq = sp + P_BYTES;
+#pragma unroll
+            for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
+                read_step((ks + 1) & 1, sp, sq, ks + 1);
+#pragma unroll
+                for (int x = 0; x < TI; ++x)
+#pragma unroll
+                    for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
+#pragma unroll
                 for (int i = 0; i < kReads; ++i) {
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // one LDS read
                     __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRead, 0);  // then MFMAs
@@ -425,33 +551,27 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             }
             constexpr int kLast = (kStepsPerSlab - 1) & 1;
             // step 3a
-    #pragma unroll
+#pragma unroll
             for (int x = 0; x < TI / 2; ++x)
-    #pragma unroll
+#pragma unroll
                 for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
-    #ifndef FMOE_DEBUG_SKIP_LDS_WRITE
             write_lds((s + 1) & 1, with_bias);
-    #endif
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < kMfma / 2; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // one MFMA
                 __builtin_amdgcn_sched_group_barrier(0x200, (NP + NQ) / (kMfma / 2), 0); // then LDS writes
             }
             __builtin_amdgcn_sched_barrier(0);
-    #ifndef FMOE_DEBUG_SKIP_BARRIER
             __syncthreads();
-    #endif
             __builtin_amdgcn_sched_barrier(0);
             // step 3b
-    #ifndef FMOE_DEBUG_SKIP_GLOBAL
-            issue_loads((s + 2) * BKE);
-    #endif
+            issue_loads((s + 2) * BKE, 0);
             read_step(0, smem + ((s + 1) & 1) * STAGE_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES + P_BYTES, 0);
-    #pragma unroll
+#pragma unroll
             for (int x = TI / 2; x < TI; ++x)
-    #pragma unroll
+#pragma unroll
                 for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < kMfma / 2; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // one MFMA
                 __builtin_amdgcn_sched_group_barrier(0x020, (NP + NQ) / (kMfma / 2), 0);  // global loads
@@ -459,6 +579,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+      }
     };
     bool want_bias = false;
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) want_bias = prm.bias_grad != nullptr && nt == 0;
@@ -471,11 +592,12 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
         if (want_bias) {
-            // thread t holds columns (t % Q_CPR) * CE .. + CE - 1 of contraction rows t / Q_CPR (mod Q_KPI);
+            // thread t holds CE columns of contraction rows t / Q_CPR (mod Q_KPI);
             // the Q_KPI partial sums of a column are added in ascending order
             float *red = (float *)smem;
             __syncthreads();
-            const int grp = t / Q_CPR, c = t % Q_CPR;
+            // the chunk this thread stages is the one that belongs in its (swizzled) slot
+            const int grp = t / Q_CPR, c = (t % Q_CPR) ^ mc_swz<T>(grp);
 #pragma unroll
             for (int j = 0; j < CE; ++j) red[grp * BM + c * CE + j] = bsum[j];
             __syncthreads();
@@ -605,6 +727,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             lds_sync();
         }
     }
+#endif  // __HIP_DEVICE_COMPILE__
 }
 
 template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI>
