@@ -98,6 +98,8 @@ def main():
     ap.add_argument("--config", default="config4", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-steps", type=int, default=3)
+    ap.add_argument("--fuse", choices=["auto", "on", "off"], default="auto",
+                    help="override the configuration's choice of the fused pipeline")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the single-GPU MoE path only; run with --gpus 1 "
@@ -107,7 +109,9 @@ def main():
     from fastermoe_amd import _lib
 
     os.environ.setdefault("FMOE_FUSE_GRAN", "4")
-    cfg = CONFIGS[args.config]
+    cfg = dict(CONFIGS[args.config])
+    if args.fuse != "auto":
+        cfg["fuse"] = args.fuse == "on"
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     device = torch.device("cuda:0")

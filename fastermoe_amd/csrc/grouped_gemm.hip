@@ -10,25 +10,12 @@
 //   dgrad    dX[seg] = dY[seg] . W_e       rows ragged, contraction = out
 //   wgrad    dW_e    = dY[seg]^T . X[seg]  contraction ragged (the segment)
 //
-// Tiling.  A 256-thread workgroup (4 waves, 2 x 2) owns a BM x BN tile of C and
-// walks the contraction in slabs of 128 bytes per row (64 bf16 / 32 fp32).
-// Both operand slabs are staged in LDS, double buffered: the global loads of
-// slab k+1 are issued before the MFMAs of slab k and written to the other LDS
-// buffer afterwards, one barrier per slab.  Each wave computes a
-// (BM/2) x (BN/2) sub-tile as 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16 /
-// _f16, v_mfma_f32_32x32x2_f32), accumulating in fp32.
-//
-// The MFMA's row index is mapped to C's COLUMN, so a lane ends up with four
-// consecutive columns of one row in adjacent accumulator registers and the
-// epilogue stores them as one 8/16-byte vector.
-//
-// Operands come in two memory shapes.  "KC": the contraction index is the
-// contiguous one (X, dY as the row operand, W in forward); the LDS slab is
-// [row][128 B] with the 16-byte chunks XOR-swizzled by the row so that the
-// 16-byte fragment reads of 32 consecutive rows spread over all banks.  "MC":
-// the row index is contiguous and the contraction strided (W in dgrad, both
-// operands in wgrad); the slab is kept as [k][rows] and the fragment is
-// collected along k when it is read.
+// This file holds the host side: segment tables, launch plans per product and per
+// chunk, the any-shape fallback kernel (feature sizes that are not a multiple of 16
+// bytes, fp64) and the stand-alone bias-gradient kernel that fallback needs.  The MFMA
+// kernel itself (tiling, LDS layouts, software pipeline, epilogues) is in
+// gemm_kernel.hpp and is instantiated once per element type and product by
+// gemm_inst.hip.
 #include "gemm_kernel.hpp"
 #include "profile.hpp"
 
