@@ -100,6 +100,9 @@ def main():
     ap.add_argument("--profile-steps", type=int, default=3)
     ap.add_argument("--fuse", choices=["auto", "on", "off"], default="auto",
                     help="override the configuration's choice of the fused pipeline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain row-copy kernel of known size (1 GiB read + 1 GiB written per launch); "
+                         "used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the single-GPU MoE path only; run with --gpus 1 "
@@ -116,6 +119,17 @@ def main():
         sys.exit("bench.py needs a GPU")
     device = torch.device("cuda:0")
     _lib.load()
+    if args.copy_calibration:
+        from fastermoe_amd import fmoe_native
+        rows, width = 131072, 4096  # bf16: 1 GiB in, 1 GiB out
+        src = torch.randn(rows, width, device=device).to(torch.bfloat16)
+        ident = torch.arange(rows, dtype=torch.int64, device=device)
+        for _ in range(5):
+            fmoe_native.gather_rows(src, ident)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "gather_rows_vec_kernel", "bytes_read": rows * width * 2,
+                          "bytes_written": rows * width * 2, "launches": 5}))
+        return
     layer, x, grad = build_layer(cfg, device)
 
     for _ in range(args.warmup):
