@@ -36,6 +36,10 @@ CONFIGS = {
 }
 
 PEAK = {"bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
+# HBM-side bytes per launch of the grouped GEMM at config 4 (rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
+# what the same counter reads for a copy kernel of known size: 1.984 and 1.000); measured offline, not in this
+# script -- the counters need their own profiler runs.
+TRAFFIC_BYTES = {"config4": {"gemm_fwd": 4.10e9, "gemm_dgrad": 4.07e9, "gemm_wgrad": 4.21e9}}
 HBM_PEAK_GBS = 8000.0
 
 
@@ -168,7 +172,7 @@ def main():
     roofline = {"kernel": "grouped_gemm_kernel (" + dominant + ")", "bound": "mfma", "achieved": round(dk["achieved"], 2),
                 "peak": peak, "unit": "TFLOP/s", "frac": round(dk["achieved"] / peak, 4),
                 "flop_per_launch": dk["work_per_launch"], "avg_launch_ms": round(dk["avg_ms"], 4),
-                "traffic": None}
+                "traffic": TRAFFIC_BYTES.get(args.config, {}).get(dominant) if cfg["fuse"] else None}
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_names)
     gemm_flop = sum(kernels[k]["work_per_launch"] * kernels[k]["launches_per_step"] for k in gemm_names)
 
