@@ -119,6 +119,7 @@ struct GemmParams {
     int32_t activation;
     int32_t accumulate_first;  // ragged-K: expert 0 of the table adds to C
     int32_t epilogue;          // Epilogue, read by the any-shape kernel only
+    int32_t block_m;           // host only: tile height the segment table was built for (256 or 128)
     int32_t profile_class;     // host only: ProfileClass of this launch
     double profile_work;       // host only: flop of this launch
     SegmentTable tab;
@@ -750,12 +751,13 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
     return FMOE_OK;
 }
 
-// Tile counts for a 256 x 256 tiling, then the launch for the requested epilogue.
-// EPI_MASK lists the epilogues a product can be asked for, so that only those
-// kernels are built.
-template <typename T, int PS, int QS, int RG, int EPI_MASK>
-int launch_by_epilogue(GemmParams &prm, int epi, hipStream_t stream) {
-    constexpr int BM = 256, BN = 256;
+// Tile counts, then the launch for the requested epilogue.  prm.block_m (256 or 128,
+// chosen by the host from the segment lengths) is the tile height; the width is 256.
+// EPI_MASK lists the epilogues a product can be asked for, so that only those kernels
+// are built.
+template <typename T, int BM, int PS, int QS, int RG, int EPI_MASK>
+int launch_for_height(GemmParams &prm, int epi, hipStream_t stream) {
+    constexpr int BN = 256;
     prm.tiles_n = (int)ceil_div(prm.n_cols, BN);
     if (RG == kRaggedRows) {
         prm.tiles_m = 0;
@@ -771,6 +773,13 @@ int launch_by_epilogue(GemmParams &prm, int epi, hipStream_t stream) {
     if constexpr ((EPI_MASK >> kEpiDAct) & 1)
         if (epi == kEpiDAct) return launch_tiles<T, BM, BN, PS, QS, RG, kEpiDAct>(prm, stream);
     return fail(FMOE_EINVAL, "epilogue %d is not built for this product", epi);
+}
+
+template <typename T, int PS, int QS, int RG, int EPI_MASK>
+int launch_by_epilogue(GemmParams &prm, int epi, hipStream_t stream) {
+    if (prm.block_m == 128) return launch_for_height<T, 128, PS, QS, RG, EPI_MASK>(prm, epi, stream);
+    if (prm.block_m == 256) return launch_for_height<T, 256, PS, QS, RG, EPI_MASK>(prm, epi, stream);
+    return fail(FMOE_EINVAL, "tile height %d is not built", prm.block_m);
 }
 
 }  // namespace gemm
