@@ -173,6 +173,32 @@ def main():
                 "peak": peak, "unit": "TFLOP/s", "frac": round(dk["achieved"] / peak, 4),
                 "flop_per_launch": dk["work_per_launch"], "avg_launch_ms": round(dk["avg_ms"], 4),
                 "traffic": TRAFFIC_BYTES.get(args.config, {}).get(dominant) if cfg["fuse"] else None}
+    # the row permutes alone (inside the fused pipeline they share the chip with the GEMMs)
+    from fastermoe_amd import fmoe_native
+    n, k, d = cfg["n"], cfg["k"], cfg["d"]
+    with torch.no_grad():
+        idx, _ = layer.gate(x)
+        cnt, pos_buf, s2r = fmoe_native.route(idx.contiguous(), cfg["e"])
+        pos = pos_buf[: int(cnt.sum())]
+        tok = pos // k
+        _lib.profile_enable(True)
+        _lib.profile_collect()
+        for _ in range(10):
+            buf = fmoe_native.gather_rows(x.detach(), tok)            # local scatter
+            fmoe_native.gather_rows(buf, s2r, n * k)                   # local gather (copy)
+        gather_alone = _lib.profile_collect()["gather_rows"]
+        for _ in range(10):
+            fmoe_native.reduce_slots(buf, s2r, n, k)                   # backward of the scatter
+        reduce_alone = _lib.profile_collect()["reduce_slots"]
+        _lib.profile_enable(False)
+    permute_alone = {
+        "gather_rows": {"GB/s": round(gather_alone[2] / gather_alone[1] / 1e6, 1),
+                        "frac_of_hbm_peak": round(gather_alone[2] / gather_alone[1] / 1e6 / HBM_PEAK_GBS, 4)},
+        "reduce_slots": {"GB/s": round(reduce_alone[2] / reduce_alone[1] / 1e6, 1),
+                         "frac_of_hbm_peak": round(reduce_alone[2] / reduce_alone[1] / 1e6 / HBM_PEAK_GBS, 4)},
+    }
+    del buf
+
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_names)
     gemm_flop = sum(kernels[k]["work_per_launch"] * kernels[k]["launches_per_step"] for k in gemm_names)
 
@@ -190,12 +216,13 @@ def main():
                      "ms_per_step": round(gemm_ms, 3)},
         "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()}
                     for k, v in kernels.items()},
+        "permute_alone": permute_alone,
         "hbm_peak_gbs": HBM_PEAK_GBS,
     }
 
     if not args.no_cpu_baseline:
         from oracle import moe as omoe
-        sample = {"config1": cfg["n"], "config4": 1024}.get(args.config, 2048)
+        sample = {"config1": cfg["n"], "config4": 4096}.get(args.config, 4096)
         sample = min(sample, cfg["n"])
         tps, cores, secs = omoe.time_cpu_baseline(sample, cfg["d"], cfg["h"], cfg["e"], cfg["k"], "gelu",
                                                   seed=1, repeats=1, threads=min(os.cpu_count() or 1, 16))

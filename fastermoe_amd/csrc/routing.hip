@@ -248,6 +248,11 @@ __global__ __launch_bounds__(kBlock) void limit_by_capacity_kernel(
     cap[e] = left;
 }
 
+__global__ __launch_bounds__(kBlock) void zero_counts_kernel(int64_t *__restrict__ count, int64_t n) {
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e < n) count[e] = 0;
+}
+
 int ilog2_ceil(int64_t n) {
     int b = 0;
     while ((1ll << b) < n) ++b;
@@ -341,7 +346,9 @@ extern "C" int fmoe_route(const int64_t *gate, int64_t n_slots, int64_t n_expert
     FMOE_REQUIRE(expert_count, "fmoe_route: NULL expert_count");
     hipStream_t st = (hipStream_t)stream;
     if (n_slots == 0) {
-        FMOE_HIP_CHECK(hipMemsetAsync(expert_count, 0, n_expert * sizeof(int64_t), st));
+        // a fill kernel, not hipMemsetAsync, so that the call can be captured into a HIP graph
+        zero_counts_kernel<<<(int)ceil_div(n_expert, kBlock), kBlock, 0, st>>>(expert_count, n_expert);
+        FMOE_LAUNCH_CHECK();
         return FMOE_OK;
     }
     FMOE_REQUIRE(gate && pos, "fmoe_route: NULL pointer");

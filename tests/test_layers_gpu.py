@@ -273,3 +273,48 @@ def test_gate_hook_and_state_dict(device):
     clone.load_state_dict(moe.state_dict())
     x = torch.rand(5, 8, device=device)
     assert torch.equal(moe(x), clone(x))
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_no_tokens(fuse, device):
+    """An empty batch goes through every kernel wrapper without a launch failing and gives
+    zero weight gradients."""
+    moe = fmoe.FMoETransformerMLP(num_expert=4, d_model=32, d_hidden=64, top_k=2).to(device)
+    moe.enable_fuse = fuse
+    x = torch.zeros(0, 32, device=device, requires_grad=True)
+    out = moe(x)
+    assert out.shape == (0, 32)
+    out.sum().backward()
+    assert x.grad.shape == (0, 32)
+    for p in moe.experts.parameters():
+        assert p.grad is not None and torch.count_nonzero(p.grad) == 0
+
+
+@pytest.mark.parametrize("chunks", ["2", "32"])
+def test_fused_many_experts_few_rows(chunks, device, monkeypatch):
+    """More experts than one launch's segment table holds (256) and more chunks than some
+    experts have rows: fused and unfused still agree, experts without rows get zero grads."""
+    monkeypatch.setenv("FMOE_FUSE_GRAN", chunks)
+    torch.manual_seed(11)
+    n, d, h, e, k = 200, 32, 48, 300, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.ReLU()).to(device)
+    x = torch.randn(n, d, device=device)
+    idx = torch.randint(0, e, (n, k), device=device)
+    score = torch.rand(n, k, device=device)
+    moe.gate.forward = lambda inp: (idx, score)
+    results = []
+    for fuse in (False, True):
+        moe.enable_fuse = fuse
+        moe.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        out.mean().backward()
+        results.append([out, xi.grad] + [p.grad.clone() for p in moe.experts.parameters()])
+    for a, b in zip(*results):
+        assert rel_err(a, b) <= 1e-5
+    used = torch.zeros(e, dtype=torch.bool, device=device)
+    used[idx.view(-1)] = True
+    assert torch.count_nonzero(moe.experts.htoh4.weight.grad[~used]) == 0
+    ref = _oracle(moe, x, idx, score, "relu", k)
+    assert rel_err(results[1][0], ref["out"]) <= 1e-5
+    assert rel_err(results[1][2], ref["grad_w1"]) <= 1e-5
