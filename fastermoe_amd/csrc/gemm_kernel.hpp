@@ -127,9 +127,11 @@ struct GemmParams {
 
 // KC slabs: 16-byte chunk c of row r is stored at chunk c ^ swz(r).
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
-// MC slabs of 16-bit elements: chunk c of contraction row k is stored at c ^ ((k % 4) * 2),
-// so that the four k rows one transposing read touches sit in different banks.
-template <typename T> __device__ __forceinline__ int mc_swz(int k) { return sizeof(T) == 2 ? (k & 3) << 1 : 0; }
+// MC slabs of 16-bit elements: chunk c of contraction row k is stored at c ^ ((k % 4) * 4).
+// A transposing read of 32 lanes touches 4 k rows x 4 chunks (two 16-column blocks); rows
+// are a multiple of 256 B apart, so without the swizzle they would share banks -- with it
+// the 16 chunks fall on the 16 distinct 16-byte positions of the 256-byte bank cycle.
+template <typename T> __device__ __forceinline__ int mc_swz(int k) { return sizeof(T) == 2 ? (k & 3) << 2 : 0; }
 
 // ---- the kernel ---------------------------------------------------------------
 template <typename T, int BM, int BN, int PSHAPE, int QSHAPE, int RAGGED, int EPI>
@@ -291,7 +293,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      :
                      : "s"(lds_addr), "v"(voff), "s"(rs)
-                     : "memory");
+                     : "memory", "m0");
     };
     u32x4 pg[NP], qg[NQ];  // register path only
 
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             const int grp = lane >> 4, s16 = lane & 15;
             const int col = r0 + (grp & 1) * 16 + 4 * (s16 & 3);
             const int kq = s16 >> 2;
-            const int chunk = (col >> 3) ^ (kq << 1);   // MC slabs are swizzled by k % 4
+            const int chunk = (col >> 3) ^ (kq << 2);   // MC slabs are swizzled by k % 4
             const int kb = ks * 16 + (grp >> 1) * 8 + kq;
             const unsigned char *base = slab + chunk * 16 + (col & 7) * 2;
             typedef short s16x4 __attribute__((ext_vector_type(4)));
