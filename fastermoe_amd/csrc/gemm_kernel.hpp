@@ -739,11 +739,15 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
     constexpr int smem_loop = 2 * (BM + BN) * kSlabBytes;
     constexpr int smem_epi = kWavesM * kWavesN * (BM / kWavesM) * (256 + 16);
     constexpr int smem = smem_loop > smem_epi ? smem_loop : smem_epi;
-    static bool configured = false;
+    // the opt-in to more than 64 KiB of dynamic LDS is per device
+    static bool configured[16] = {};
     auto kern = grouped_gemm_kernel<T, BM, BN, PS, QS, RG, EPI>;
-    if (!configured) {
+    int dev = 0;
+    FMOE_HIP_CHECK(hipGetDevice(&dev));
+    FMOE_REQUIRE(dev >= 0 && dev < 16, "device index %d out of range", dev);
+    if (!configured[dev]) {
         FMOE_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured = true;
+        configured[dev] = true;
     }
     if (prm.total_tiles <= 0) return FMOE_OK;
     const int grid = (prm.total_tiles + 7) / 8 * 8;
@@ -761,13 +765,16 @@ template <typename T, int BM, int PS, int QS, int RG, int EPI_MASK>
 int launch_for_height(GemmParams &prm, int epi, hipStream_t stream) {
     constexpr int BN = 256;
     prm.tiles_n = (int)ceil_div(prm.n_cols, BN);
+    int64_t total;
     if (RG == kRaggedRows) {
         prm.tiles_m = 0;
-        prm.total_tiles = prm.tab.tile[prm.tab.n] * prm.tiles_n;
+        total = (int64_t)prm.tab.tile[prm.tab.n] * prm.tiles_n;
     } else {
         prm.tiles_m = (int)ceil_div(prm.n_rows, BM);
-        prm.total_tiles = prm.tab.n * prm.tiles_m * prm.tiles_n;
+        total = (int64_t)prm.tab.n * prm.tiles_m * prm.tiles_n;
     }
+    if (total > (int64_t)INT32_MAX - 8) return fail(FMOE_ELIMIT, "grouped GEMM: %lld tiles exceed the grid limit", (long long)total);
+    prm.total_tiles = (int)total;
     if constexpr ((EPI_MASK >> kEpiStore) & 1)
         if (epi == kEpiStore) return launch_tiles<T, BM, BN, PS, QS, RG, kEpiStore>(prm, stream);
     if constexpr ((EPI_MASK >> kEpiBiasAct) & 1)

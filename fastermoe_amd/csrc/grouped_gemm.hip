@@ -210,8 +210,10 @@ template <typename T> bool fast_ok(std::initializer_list<const void *> ptrs, std
     constexpr int CE = 16 / (int)sizeof(T);
     for (const void *p : ptrs)
         if (p && !aligned16(p)) return false;
+    // a row must be a whole number of 16-byte chunks, and 256 rows must stay inside the
+    // 2 GiB a buffer offset can address
     for (int64_t d : dims)
-        if (d % CE != 0) return false;
+        if (d % CE != 0 || d * (int64_t)sizeof(T) > (int64_t)(1 << 22)) return false;
     return true;
 }
 
