@@ -222,7 +222,7 @@ def main():
 
     if not args.no_cpu_baseline:
         from oracle import moe as omoe
-        sample = {"config1": cfg["n"], "config4": 4096}.get(args.config, 4096)
+        sample = {"config1": cfg["n"], "config4": 8192}.get(args.config, 4096)
         sample = min(sample, cfg["n"])
         tps, cores, secs = omoe.time_cpu_baseline(sample, cfg["d"], cfg["h"], cfg["e"], cfg["k"], "gelu",
                                                   seed=1, repeats=1, threads=min(os.cpu_count() or 1, 16))

@@ -134,6 +134,20 @@ inline char *at(void *base, int64_t row, int64_t row_elems, int dtype) {
 
 using namespace fmoe;
 
+extern "C" int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert, int n_chunks,
+                                       int64_t *bounds_host) {
+    FMOE_REQUIRE(expert_count_host && bounds_host && n_expert >= 1, "fmoe_fused_chunk_bounds: bad argument");
+    FMOE_REQUIRE(n_chunks >= 1 && n_chunks <= kMaxChunks, "fmoe_fused_chunk_bounds: n_chunks=%d (1..%d)", n_chunks,
+                 kMaxChunks);
+    int64_t rows = 0;
+    for (int64_t e = 0; e < n_expert; ++e) {
+        FMOE_REQUIRE(expert_count_host[e] >= 0, "fmoe_fused_chunk_bounds: negative expert count");
+        rows += expert_count_host[e];
+    }
+    chunk_bounds(expert_count_host, n_expert, rows, n_chunks, bounds_host);
+    return FMOE_OK;
+}
+
 extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp, const int64_t *pos,
                                       const int64_t *slot_to_row, const int64_t *expert_count_host,
                                       int64_t n_tokens, int64_t top_k, int64_t n_rows, void *buf_in,

@@ -178,6 +178,14 @@ typedef struct fmoe_mlp_params {
     int activation;   /* FMOE_ACT_* */
 } fmoe_mlp_params;
 
+/* Row bounds of the pipeline's chunks: chunk c covers the expert-sorted rows
+ * [bounds_host[c], bounds_host[c+1]), bounds_host has n_chunks + 1 entries.
+ * The split is even except that a bound moves to an expert boundary lying
+ * within a quarter chunk of it.  Host only, no GPU work.  Plays the part of
+ * the worker-group stepping of cuda/fused_compute.cuh:276-280. */
+int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert,
+                            int n_chunks, int64_t *bounds_host);
+
 /* Forward of scatter -> Linear -> act -> Linear -> gather over `n_chunks`
  * contiguous chunks of the expert-sorted rows, chunk c+1's scatter and chunk
  * c-1's gather running beside chunk c's GEMMs on the library's own streams,

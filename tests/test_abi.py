@@ -126,3 +126,35 @@ def test_activation_codes():
         _activation_code(torch.nn.GELU(approximate="tanh"))
     with pytest.raises(NotImplementedError):
         _activation_code(torch.nn.Tanh())
+
+
+def test_fused_chunk_bounds_host_logic():
+    """Chunk planning of the fused pipeline (host only): monotone, covers all rows, snaps to an
+    expert boundary within a quarter chunk, otherwise splits evenly."""
+    import ctypes
+    lib = _lib.load()
+
+    def bounds(counts, n_chunks):
+        c = (ctypes.c_int64 * len(counts))(*counts)
+        b = (ctypes.c_int64 * (n_chunks + 1))()
+        _lib.check(lib.fmoe_fused_chunk_bounds(ctypes.cast(c, ctypes.c_void_p), len(counts), n_chunks,
+                                               ctypes.cast(b, ctypes.c_void_p)))
+        return list(b)
+
+    # 8 nearly equal experts, 4 chunks: every bound lands on an expert boundary
+    counts = [8100, 8300, 8192, 8000, 8400, 8192, 8150, 8202]
+    b = bounds(counts, 4)
+    prefix = [sum(counts[:i]) for i in range(9)]
+    assert b[0] == 0 and b[-1] == sum(counts) and all(x in prefix for x in b)
+    # one huge expert: no boundary nearby, even split
+    assert bounds([1000], 4) == [0, 250, 500, 750, 1000]
+    # boundary too far from the even split stays even
+    assert bounds([100, 900], 2) == [0, 500, 1000]
+    # boundary within a quarter chunk is taken
+    assert bounds([450, 550], 2) == [0, 450, 1000]
+    # more chunks than rows, empty experts: still monotone and complete
+    b = bounds([0, 3, 0, 0, 2], 8)
+    assert b[0] == 0 and b[-1] == 5 and all(x <= y for x, y in zip(b, b[1:]))
+    assert bounds([0, 0], 3) == [0, 0, 0, 0]
+    rc = lib.fmoe_fused_chunk_bounds(None, 2, 3, None)
+    assert rc == -1
