@@ -149,22 +149,28 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     // -- which tile ------------------------------------------------------------
-    const int per_xcd = (gridDim.x + 7) >> 3;
-    const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (L >= prm.total_tiles) return;
-
+    // Workgroup b runs on XCD b % 8 (each XCD has its own L2).  Ragged rows: tiles cost the
+    // same, so every XCD takes a contiguous eighth of the logical tile order.  Ragged K: a
+    // tile costs as much as its expert has rows, so every XCD takes a contiguous eighth of
+    // EACH expert's tiles instead -- skewed routing then loads the XCDs evenly.
     int ei, mt, nt;
     {
         int tm_total, rem;
         if (RAGGED == kRaggedRows) {
+            const int per_xcd = (gridDim.x + 7) >> 3;
+            const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+            if (L >= prm.total_tiles) return;
             tm_total = prm.tab.tile[prm.tab.n];
             rem = L;
             ei = 0;
         } else {
             const int tpe = prm.tiles_m * prm.tiles_n;
+            const int share = (tpe + 7) >> 3;  // tiles of one expert per XCD
+            const int i = blockIdx.x >> 3;
             tm_total = prm.tiles_m;
-            ei = L / tpe;
-            rem = L - ei * tpe;
+            ei = i / share;
+            rem = (blockIdx.x & 7) * share + (i - ei * share);
+            if (ei >= prm.tab.n || rem >= tpe) return;
         }
         const int gspan = kGroupM * prm.tiles_n;
         const int grp = rem / gspan;
@@ -214,6 +220,21 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     const int lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     const int wave_m0 = (wave / kWavesN) * WM, wave_n0 = (wave % kWavesN) * WN;
+
+    // An expert without rows has a zero weight gradient (and bias gradient): write the
+    // tile with plain coalesced stores and skip the whole pipeline.
+    if constexpr (RAGGED == kRaggedK) {
+        if (K == 0) {
+            constexpr int kChunksPerRow = BN / CE;
+            for (int q = t; q < BM * kChunksPerRow; q += kThreads) {
+                const int r = q / kChunksPerRow, c = q % kChunksPerRow;
+                if (r < q_valid && c * CE < p_valid) *(u32x4 *)(Cb + (int64_t)r * prm.ldc + c * CE) = u32x4{0, 0, 0, 0};
+            }
+            if (prm.bias_grad != nullptr && nt == 0 && t < q_valid)
+                ((T *)prm.bias_grad)[(int64_t)expert * prm.n_rows + mt * BM + t] = (T)0.f;
+            return;
+        }
+    }
 
     // -- global -> register -> LDS staging ---------------------------------------
     // Loads go through buffer instructions: an offset at or beyond the resource's
@@ -750,7 +771,13 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
         configured[dev] = true;
     }
     if (prm.total_tiles <= 0) return FMOE_OK;
-    const int grid = (prm.total_tiles + 7) / 8 * 8;
+    // ragged rows: the tiles rounded up to a multiple of 8; ragged K: 8 XCDs x experts x an
+    // eighth (rounded up) of one expert's tiles -- the kernel drops the surplus workgroups
+    const int64_t grid64 = (RG == kRaggedRows)
+                               ? ((int64_t)prm.total_tiles + 7) / 8 * 8
+                               : (int64_t)8 * prm.tab.n * (((int64_t)prm.tiles_m * prm.tiles_n + 7) / 8);
+    if (grid64 > (int64_t)INT32_MAX) return fail(FMOE_ELIMIT, "grouped GEMM: grid of %lld workgroups", (long long)grid64);
+    const int grid = (int)grid64;
     ProfileScope prof(prm.profile_class, prm.profile_work, stream);
     kern<<<grid, kThreads, smem, stream>>>(prm);
     FMOE_LAUNCH_CHECK();
