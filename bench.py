@@ -107,6 +107,10 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain row-copy kernel of known size (1 GiB read + 1 GiB written per launch); "
                          "used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--reference-gemm", action="store_true",
+                    help="time one expert's forward GEMM of the workload (rows/experts x d_model x d_hidden) with the "
+                         "grouped kernel and with the vendor library (torch.nn.functional.linear), on N(0,1) and on "
+                         "all-zero operands; shows how much of the datasheet peak the power envelope leaves")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the single-GPU MoE path only; run with --gpus 1 "
@@ -133,6 +137,36 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "gather_rows_vec_kernel", "bytes_read": rows * width * 2,
                           "bytes_written": rows * width * 2, "launches": 5}))
+        return
+    if args.reference_gemm:
+        from fastermoe_amd import fmoe_native
+        dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+        rows = cfg["n"] * cfg["k"] // cfg["e"]
+        cnt = torch.tensor([rows], dtype=torch.int64)
+
+        def timed(fn, iters=10):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(iters):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / iters
+
+        out = {"shape": [rows, cfg["d"], cfg["h"]], "dtype": cfg["dtype"], "unit": "TFLOP/s"}
+        flop = 2.0 * rows * cfg["d"] * cfg["h"]
+        for name in ("normal", "zeros"):
+            xx = torch.randn(rows, cfg["d"], device=device).to(dtype)
+            ww = torch.randn(1, cfg["h"], cfg["d"], device=device).to(dtype)
+            if name == "zeros":
+                xx.zero_()
+                ww.zero_()
+            out["grouped_kernel_" + name] = round(flop / timed(lambda: fmoe_native.linear_forward(xx, cnt, ww, None)) / 1e9, 1)
+            out["vendor_library_" + name] = round(flop / timed(lambda: torch.nn.functional.linear(xx, ww[0])) / 1e9, 1)
+        print(json.dumps(out))
         return
     layer, x, grad = build_layer(cfg, device)
 

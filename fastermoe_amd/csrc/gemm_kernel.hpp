@@ -25,10 +25,6 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #ifndef FMOE_GEMM_WAVES_M
 #define FMOE_GEMM_WAVES_M 4
 #endif
-// 1: global loads write LDS directly (buffer_load ... lds); 0: through registers
-#ifndef FMOE_GEMM_LDS_DMA
-#define FMOE_GEMM_LDS_DMA 1
-#endif
 constexpr int kWavesM = FMOE_GEMM_WAVES_M, kWavesN = 2;
 constexpr int kThreads = 64 * kWavesM * kWavesN;
 constexpr int kRowsPerPass = kThreads / 8;  // KC slabs: rows covered by one 16-byte load of every thread
@@ -144,7 +140,6 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int NP = BN * 8 / kThreads;            // 16-byte chunks per thread per slab
     constexpr int NQ = BM * 8 / kThreads;
     constexpr int P_BYTES = BN * kSlabBytes, Q_BYTES = BM * kSlabBytes;
-    constexpr int STAGE_BYTES = P_BYTES + Q_BYTES;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -236,17 +231,24 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         }
     }
 
-    // -- global -> register -> LDS staging ---------------------------------------
-    // Loads go through buffer instructions: an offset at or beyond the resource's
-    // size returns zeros, so rows outside the tile and the contraction tail need no
-    // branch -- their offset is replaced by kOutOfRange.
-    // KC: chunk q = it*256 + t covers row q/8, 16-byte chunk q%8 of the slab.
-    // MC: chunk q covers contraction row q / CPR, 16-byte column chunk q % CPR.
+    // -- global -> LDS staging ------------------------------------------------------
+    // Slabs go from memory straight into LDS (buffer_load ... lds: lane i of a wave lands
+    // at base + 16 i).  An offset at or beyond the buffer resource's size returns zeros, so
+    // rows outside the tile and the contraction tail need no branch -- their offset is
+    // replaced by kOutOfRange and the lanes land as zeros.
+    //
+    // LDS holds three buffers for P slabs followed by two for Q slabs (160 KiB at 256 x 256).
+    // While slab s is computed from, slab s+1 is complete or landing, the P part of slab s+2
+    // is requested at the start of slab s and its Q part right after the barrier that ends
+    // slab s: the loads are spread over the slab (a burst of them would fill the load
+    // queue and block the MFMAs behind it) and the P loads have more than a slab to land.
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
     constexpr int P_CPR = BN / CE, P_KPI = kThreads / P_CPR;  // MC: chunks per k row, k rows per pass
     constexpr int Q_CPR = BM / CE, Q_KPI = kThreads / Q_CPR;
     constexpr int kPassBytes = kThreads * 16;  // LDS bytes filled by one 16-byte load of every thread
+    constexpr int kPBufs = 3;
+    constexpr int Q_BASE = kPBufs * P_BYTES;
 
     // Slot q = it*kThreads + t of a slab is filled by thread t in pass it, so a wave fills
     // 1 KiB of consecutive LDS per load.  The swizzle is applied on the memory side: the
@@ -288,15 +290,12 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                              : kOutOfRange;
     }
 
-    // Direct-to-LDS loads pay off when both slabs are KC (forward); with an MC slab the
-    // register path measured faster, so the choice is per product.
-    constexpr bool kDma = FMOE_GEMM_LDS_DMA != 0;
     // With an MC slab the fragments are read by ds_read_b64_tr_b16, and the compiler puts a
     // full vmcnt(0) wait between a direct-to-LDS load and any such read that follows it
-    // (it cannot tell the two LDS buffers apart), which would serialise the pipeline.  For
+    // (it cannot tell the LDS buffers apart), which would serialise the pipeline.  For
     // those products the load is emitted as inline assembly, which the compiler does not
-    // track; the one wait that is needed (before the barrier) is written out by hand.
-    constexpr bool kDmaAsm = kDma && (PSHAPE == kMC || QSHAPE == kMC);
+    // track; the waits that are needed (before the barriers) are written out by hand.
+    constexpr bool kDmaAsm = (PSHAPE == kMC || QSHAPE == kMC);
     typedef int i32x4 __attribute__((ext_vector_type(4)));
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)smem;
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -316,56 +315,39 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                      : "s"(lds_addr), "v"(voff), "s"(rs)
                      : "memory", "m0");
     };
-    u32x4 pg[NP], qg[NQ];  // register path only
 
-    // KC: the resource starts at contraction index k0 of the tile's first row and the
-    // chunk is dropped when it lies past K.  MC: the resource starts at contraction row
+    // One operand's part of the slab that starts at contraction index k0, into LDS offset
+    // lds_off.  KC: the resource starts at contraction index k0 of the tile's first row and
+    // the chunk is dropped when it lies past K.  MC: the resource starts at contraction row
     // k0 and is exactly as long as the rows that remain, so rows past K read as zero.
-    // With FMOE_GEMM_LDS_DMA the loads write LDS directly (buffer_load ... lds: lane i of
-    // a wave lands at base + 16 i, out-of-range lanes land as zeros) into buffer `stage`;
-    // otherwise they return in registers and write_lds() stores them.
-    auto issue_loads = [&](int k0, int stage) {
+    auto issue_part = [&](auto shape_tag, const T *tile, int64_t ld, int kc_chunk, const uint32_t *voff, auto n_tag, int k0,
+                          uint32_t lds_off) {
+        constexpr int SHAPE = decltype(shape_tag)::value;
+        constexpr int N = decltype(n_tag)::value;
         const int k_left = K - k0;  // <= 0 past the end: everything reads as zero
-        unsigned char *sp = smem + stage * STAGE_BYTES + wave * 1024;
-        unsigned char *sq = sp + P_BYTES;
-        (void)sp; (void)sq;
-        {
-            const T *origin = (PSHAPE == kKC) ? Pb + k0 : Pb + (int64_t)k0 * prm.ldp;
-            int64_t bytes = (PSHAPE == kKC) ? (int64_t)kOutOfRange : (int64_t)k_left * prm.ldp * (int64_t)sizeof(T);
-            bytes = bytes < 0 ? 0 : (bytes > (int64_t)kOutOfRange ? (int64_t)kOutOfRange : bytes);
-            const __amdgpu_buffer_rsrc_t rsrc =
-                __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
-            // sign bit of (k_left - 1 - first k of the chunk): set exactly when the chunk starts past K
-            const uint32_t past = (PSHAPE == kKC) ? ((uint32_t)(k_left - 1 - p_kc_chunk * CE) & kOutOfRange) : 0u;
+        const T *origin = (SHAPE == kKC) ? tile + k0 : tile + (int64_t)k0 * ld;
+        int64_t bytes = (SHAPE == kKC) ? (int64_t)kOutOfRange : (int64_t)k_left * ld * (int64_t)sizeof(T);
+        bytes = bytes < 0 ? 0 : (bytes > (int64_t)kOutOfRange ? (int64_t)kOutOfRange : bytes);
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
+        // sign bit of (k_left - 1 - first k of the chunk): set exactly when the chunk starts past K
+        const uint32_t past = (SHAPE == kKC) ? ((uint32_t)(k_left - 1 - kc_chunk * CE) & kOutOfRange) : 0u;
 #pragma unroll
-            for (int it = 0; it < NP; ++it) {
-                if constexpr (kDmaAsm)
-                    dma_asm(origin, bytes, stage * STAGE_BYTES + wave_u * 1024 + it * kPassBytes, p_voff[it] | past);
-                else if constexpr (kDma)
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(sp + it * kPassBytes),
-                                                             16, p_voff[it] | past, 0, 0, 0);
-                else
-                    pg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, p_voff[it] | past, 0, 0);
-            }
+        for (int it = 0; it < N; ++it) {
+            if constexpr (kDmaAsm)
+                dma_asm(origin, bytes, lds_off + wave_u * 1024 + it * kPassBytes, voff[it] | past);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    rsrc, (__attribute__((address_space(3))) void *)(smem + lds_off + wave * 1024 + it * kPassBytes), 16,
+                    voff[it] | past, 0, 0, 0);
         }
-        {
-            const T *origin = (QSHAPE == kKC) ? Qb + k0 : Qb + (int64_t)k0 * prm.ldq;
-            int64_t bytes = (QSHAPE == kKC) ? (int64_t)kOutOfRange : (int64_t)k_left * prm.ldq * (int64_t)sizeof(T);
-            bytes = bytes < 0 ? 0 : (bytes > (int64_t)kOutOfRange ? (int64_t)kOutOfRange : bytes);
-            const __amdgpu_buffer_rsrc_t rsrc =
-                __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
-            const uint32_t past = (QSHAPE == kKC) ? ((uint32_t)(k_left - 1 - q_kc_chunk * CE) & kOutOfRange) : 0u;
-#pragma unroll
-            for (int it = 0; it < NQ; ++it) {
-                if constexpr (kDmaAsm)
-                    dma_asm(origin, bytes, stage * STAGE_BYTES + P_BYTES + wave_u * 1024 + it * kPassBytes, q_voff[it] | past);
-                else if constexpr (kDma)
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(sq + it * kPassBytes),
-                                                             16, q_voff[it] | past, 0, 0, 0);
-                else
-                    qg[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, q_voff[it] | past, 0, 0);
-            }
-        }
+    };
+    auto issue_p = [&](int k0, int buf) {
+        issue_part(std::integral_constant<int, PSHAPE>{}, Pb, prm.ldp, p_kc_chunk, p_voff, std::integral_constant<int, NP>{}, k0,
+                   (uint32_t)(buf * P_BYTES));
+    };
+    auto issue_q = [&](int k0, int buf) {
+        issue_part(std::integral_constant<int, QSHAPE>{}, Qb, prm.ldq, q_kc_chunk, q_voff, std::integral_constant<int, NQ>{}, k0,
+                   (uint32_t)(Q_BASE + buf * Q_BYTES));
     };
 
     // Bias gradient (weight-gradient product only): the workgroups of the first column
@@ -393,27 +375,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             }
         }
     };
-
-    // Registers -> LDS (register path), or nothing (the loads wrote LDS themselves); in
-    // both cases the bias-gradient workgroups add up the chunks this thread staged.
-    auto write_lds = [&](int stage, auto with_bias) {
-        unsigned char *sp = smem + stage * STAGE_BYTES + t * 16;
-        unsigned char *sq = sp + P_BYTES;
-        if constexpr (kDma) {
-            if constexpr (decltype(with_bias)::value) {
+    // adds up the chunks this thread's loads put into Q buffer `buf` (after they have landed)
+    auto add_q_chunks = [&](int buf) {
+        const unsigned char *sq = smem + Q_BASE + buf * Q_BYTES + t * 16;
 #pragma unroll
-                for (int it = 0; it < NQ; ++it) add_chunk(*(const u32x4 *)(sq + it * kPassBytes));
-            }
-        } else {
-#pragma unroll
-            for (int it = 0; it < NP; ++it) *(u32x4 *)(sp + it * kPassBytes) = pg[it];
-#pragma unroll
-            for (int it = 0; it < NQ; ++it) *(u32x4 *)(sq + it * kPassBytes) = qg[it];
-            if constexpr (decltype(with_bias)::value) {
-#pragma unroll
-                for (int it = 0; it < NQ; ++it) add_chunk(qg[it]);
-            }
-        }
+        for (int it = 0; it < NQ; ++it) add_chunk(*(const u32x4 *)(sq + it * kPassBytes));
     };
 
     // -- fragments ---------------------------------------------------------------
@@ -459,22 +425,21 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[x][y][r] = 0.f;
 
-    // Main loop, one basic block per slab, software-pipelined by hand:
-    //   steps 0..2 : MFMAs of step ks, with the LDS reads of step ks+1 between them
-    //   step 3a    : first half of the MFMAs; the slab prefetched one iteration ago is
-    //                written to the other LDS buffer
-    //   barrier
-    //   step 3b    : second half of the MFMAs; the global loads of the slab after next
-    //                are issued and step 0 of the next slab is read from the other buffer
-    // so a global load has a whole slab of MFMAs to complete and no LDS read is waited
-    // for at the top of an iteration.  Past the last slab the loads return zeros and the
-    // extra LDS write lands in the buffer nobody reads, which keeps the body branch-free.
-    constexpr int kReadsPerFrag = (sizeof(T) == 2) ? 1 : 1;
-    constexpr int kPReads = TI * ((PSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : kReadsPerFrag);
-    constexpr int kQReads = TJ * ((QSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : kReadsPerFrag);
+    // Main loop, one basic block per slab, software-pipelined by hand.  P buffer pc holds
+    // slab s, pn slab s+1, pf receives slab s+2; Q buffer s%2 holds slab s.  Per slab:
+    //   step 0     : MFMAs of step 0, LDS reads of step 1, and the P loads of slab s+2
+    //   steps 1..2 : MFMAs of step ks, LDS reads of step ks+1 between them
+    //   step 3a    : first half of the last step's MFMAs, then wait until this wave's loads
+    //                of slab s+1 have landed (the P loads of slab s+2 stay in flight)
+    //   barrier    : slab s+1 is complete and nobody reads slab s any more
+    //   step 3b    : second half of the MFMAs; the Q part of slab s+2 is requested into the
+    //                Q buffer of slab s and step 0 of slab s+1 is read
+    // so no LDS read is waited for at the top of an iteration.  Past the last slab the
+    // loads return zeros and land in buffers nobody reads, which keeps the body branch-free.
+    constexpr int kPReads = TI * ((PSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1);
+    constexpr int kQReads = TJ * ((QSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1);
     constexpr int kReads = kPReads + kQReads;                   // LDS read instructions per step
     constexpr int kMfma = TI * TJ * (sizeof(T) == 4 ? 4 : 1);   // MFMA instructions per step
-    constexpr int kMfmaPerRead = 1;  // reads go out early in the step, the remaining MFMAs follow
 
     const int n_slabs = (K + BKE - 1) / BKE;
     u32x4 pf[2][TI], qf[2][TJ];
@@ -484,40 +449,52 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
         for (int y = 0; y < TJ; ++y) qf[buf][y] = frag(sq, QSHAPE, BM, wave_m0 + y * 32, ks);
     };
+    // s_waitcnt vmcnt(n) lgkmcnt(0): at most n of this wave's loads still in flight, all LDS reads done
+    auto wait_loads = [&](auto n_tag) {
+        constexpr int n = decltype(n_tag)::value;
+        static_assert(n < 64, "vmcnt is a 6-bit field");
+        __builtin_amdgcn_s_waitcnt(0x0070 | (n & 15) | ((n >> 4) << 14));
+    };
+    // LDS reads are complete (waited for above) when a wave arrives, so the barrier alone
+    // orders them against the loads that overwrite the buffer afterwards
+    auto slab_barrier = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
 
     auto main_loop = [&](auto with_bias) {
-      if constexpr (kDma) {
-        // Direct-to-LDS pipeline.  Buffer A = s&1 is computed from, buffer B = the other
-        // one holds (or is receiving) slab s+1.  Per slab:
-        //   steps 0..2 : MFMAs of step ks, LDS reads of step ks+1 between them
-        //   step 3a    : first half of the last step's MFMAs, then wait for this wave's
-        //                loads of slab s+1
-        //   barrier    : slab s+1 is complete in B and nobody reads A any more
-        //   step 3b    : second half of the MFMAs; slab s+2 is requested into A and
-        //                step 0 of slab s+1 is read from B
-        constexpr int kVmcnt0 = 0x0F70;  // s_waitcnt vmcnt(0), other counters untouched
-        issue_loads(0, 0);
-        __builtin_amdgcn_s_waitcnt(kVmcnt0);
-        __syncthreads();
-        if constexpr (decltype(with_bias)::value) write_lds(0, with_bias);
-        issue_loads(BKE, 1);
-        read_step(0, smem, smem + P_BYTES, 0);
+        constexpr bool kBias = decltype(with_bias)::value;
+        issue_p(0, 0);
+        issue_q(0, 0);
+        issue_p(BKE, 1);
+        issue_q(BKE, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        wait_loads(std::integral_constant<int, NP + NQ>{});  // slab 0 has landed
+        slab_barrier();
+        if constexpr (kBias) add_q_chunks(0);
+        read_step(0, smem, smem + Q_BASE, 0);
         __builtin_amdgcn_sched_barrier(0);
 
+        int pc = 0;
         for (int s = 0; s < n_slabs; ++s) {
-            const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
-            const unsigned char *sq = sp + P_BYTES;
+            const int pn = pc == kPBufs - 1 ? 0 : pc + 1;
+            const int pf_buf = pn == kPBufs - 1 ? 0 : pn + 1;
+            const unsigned char *sp = smem + pc * P_BYTES;
+            const unsigned char *sq = smem + Q_BASE + (s & 1) * Q_BYTES;
 #pragma unroll
             for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
+                if (ks == 0) issue_p((s + 2) * BKE, pf_buf);
                 read_step((ks + 1) & 1, sp, sq, ks + 1);
 #pragma unroll
                 for (int x = 0; x < TI; ++x)
 #pragma unroll
                     for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
 #pragma unroll
-                for (int i = 0; i < kReads; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRead, 0);
+                for (int i = 0; i < kMfma; ++i) {
+                    if (i < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one MFMA
+                    if (ks == 0 && i < NP) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -527,12 +504,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
                 for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
             __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_waitcnt(kVmcnt0);
-            __syncthreads();
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (decltype(with_bias)::value) write_lds((s + 1) & 1, with_bias);
-            issue_loads((s + 2) * BKE, s & 1);
-            read_step(0, smem + ((s + 1) & 1) * STAGE_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES + P_BYTES, 0);
+            wait_loads(std::integral_constant<int, NP>{});  // everything but the P loads of slab s+2
+            slab_barrier();
+            if constexpr (kBias) add_q_chunks((s + 1) & 1);
+            issue_q((s + 2) * BKE, s & 1);
+            read_step(0, smem + pn * P_BYTES, smem + Q_BASE + ((s + 1) & 1) * Q_BYTES, 0);
 #pragma unroll
             for (int x = TI / 2; x < TI; ++x)
 #pragma unroll
@@ -540,70 +516,15 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
             for (int i = 0; i < kMfma / 2; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, (NQ + kMfma / 2 - 1) / (kMfma / 2), 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma / 2 - 1) / (kMfma / 2), 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, (NP + NQ) / (kMfma / 2), 0);
             }
             __builtin_amdgcn_sched_barrier(0);
+            pc = pn;
         }
         // the loads requested past the last slab (all out of range) must land before LDS is reused
-        __builtin_amdgcn_s_waitcnt(kVmcnt0);
-        __syncthreads();
-      } else {
-        issue_loads(0, 0);
-        write_lds(0, with_bias);
-        __syncthreads();
-        issue_loads(BKE, 0);
-        read_step(0, smem, smem + P_BYTES, 0);
-        __builtin_amdgcn_sched_barrier(0);
-
-        for (int s = 0; s < n_slabs; ++s) {
-            const unsigned char *sp = smem + (s & 1) * STAGE_BYTES;
-            const unsigned char *sq = sp + P_BYTES;
-#pragma unroll
-            for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
-                read_step((ks + 1) & 1, sp, sq, ks + 1);
-#pragma unroll
-                for (int x = 0; x < TI; ++x)
-#pragma unroll
-                    for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
-#pragma unroll
-                for (int i = 0; i < kReads; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // one LDS read
-                    __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRead, 0);  // then MFMAs
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            constexpr int kLast = (kStepsPerSlab - 1) & 1;
-            // step 3a
-#pragma unroll
-            for (int x = 0; x < TI / 2; ++x)
-#pragma unroll
-                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
-            write_lds((s + 1) & 1, with_bias);
-#pragma unroll
-            for (int i = 0; i < kMfma / 2; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // one MFMA
-                __builtin_amdgcn_sched_group_barrier(0x200, (NP + NQ) / (kMfma / 2), 0); // then LDS writes
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            __syncthreads();
-            __builtin_amdgcn_sched_barrier(0);
-            // step 3b
-            issue_loads((s + 2) * BKE, 0);
-            read_step(0, smem + ((s + 1) & 1) * STAGE_BYTES, smem + ((s + 1) & 1) * STAGE_BYTES + P_BYTES, 0);
-#pragma unroll
-            for (int x = TI / 2; x < TI; ++x)
-#pragma unroll
-                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
-#pragma unroll
-            for (int i = 0; i < kMfma / 2; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // one MFMA
-                __builtin_amdgcn_sched_group_barrier(0x020, (NP + NQ) / (kMfma / 2), 0);  // global loads
-                __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma / 2 - 1) / (kMfma / 2), 0);  // LDS reads
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-      }
+        wait_loads(std::integral_constant<int, 0>{});
+        slab_barrier();
     };
     bool want_bias = false;
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) want_bias = prm.bias_grad != nullptr && nt == 0;
@@ -756,8 +677,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 
 template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI>
 int launch_tiles(GemmParams &prm, hipStream_t stream) {
-    // two slab buffers, or the epilogue's staging area (one [rows][256 B + 16 B] block per wave)
-    constexpr int smem_loop = 2 * (BM + BN) * kSlabBytes;
+    // three P and two Q slab buffers, or the epilogue's staging area (one [rows][256 B + 16 B] block per wave)
+    constexpr int smem_loop = (3 * BN + 2 * BM) * kSlabBytes;
     constexpr int smem_epi = kWavesM * kWavesN * (BM / kWavesM) * (256 + 16);
     constexpr int smem = smem_loop > smem_epi ? smem_loop : smem_epi;
     // the opt-in to more than 64 KiB of dynamic LDS is per device
