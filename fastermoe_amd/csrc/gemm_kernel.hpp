@@ -27,7 +27,15 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #endif
 constexpr int kWavesM = FMOE_GEMM_WAVES_M, kWavesN = 2;
 constexpr int kThreads = 64 * kWavesM * kWavesN;
-constexpr int kRowsPerPass = kThreads / 8;  // KC slabs: rows covered by one 16-byte load of every thread
+// The first kLoadWaves waves of a workgroup request the slabs.  The SIMD issues from its
+// oldest wave first, so with two waves per SIMD the younger one falls behind; leaving the
+// loads (which can block at a full load queue) to the older waves evens the two out.
+#ifndef FMOE_X_LOADWAVES
+#define FMOE_X_LOADWAVES 4
+#endif
+constexpr int kLoadWaves = FMOE_X_LOADWAVES;
+constexpr int kLoaders = 64 * kLoadWaves;
+constexpr int kRowsPerPass = kLoaders / 8;  // KC slabs: rows covered by one 16-byte load of every loading thread
 constexpr int kSlabBytes = 128;  // contraction bytes per row per slab
 constexpr int kStepsPerSlab = 4; // 32-byte contraction steps (two 16-byte chunks) per slab
 constexpr int kGroupM = 8;       // row tiles that share a column tile consecutively
@@ -129,6 +137,9 @@ __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 // the 16 chunks fall on the 16 distinct 16-byte positions of the 256-byte bank cycle.
 template <typename T> __device__ __forceinline__ int mc_swz(int k) { return sizeof(T) == 2 ? (k & 3) << 2 : 0; }
 
+#ifdef FMOE_X_TIMING
+__device__ unsigned long long fmoe_dbg[8 * 16384];
+#endif
 // ---- the kernel ---------------------------------------------------------------
 template <typename T, int BM, int BN, int PSHAPE, int QSHAPE, int RAGGED, int EPI>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
@@ -137,8 +148,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int BKE = kSlabBytes / (int)sizeof(T); // elements per slab row
     constexpr int WM = BM / kWavesM, WN = BN / kWavesN;  // wave tile
     constexpr int TI = WN / 32, TJ = WM / 32;        // MFMA blocks per wave (cols, rows)
-    constexpr int NP = BN * 8 / kThreads;            // 16-byte chunks per thread per slab
-    constexpr int NQ = BM * 8 / kThreads;
+    constexpr int NP = BN * 8 / kLoaders;            // 16-byte chunks per loading thread per slab
+    constexpr int NQ = BM * 8 / kLoaders;
     constexpr int P_BYTES = BN * kSlabBytes, Q_BYTES = BM * kSlabBytes;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -244,13 +255,13 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // queue and block the MFMAs behind it) and the P loads have more than a slab to land.
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
-    constexpr int P_CPR = BN / CE, P_KPI = kThreads / P_CPR;  // MC: chunks per k row, k rows per pass
-    constexpr int Q_CPR = BM / CE, Q_KPI = kThreads / Q_CPR;
-    constexpr int kPassBytes = kThreads * 16;  // LDS bytes filled by one 16-byte load of every thread
+    constexpr int P_CPR = BN / CE, P_KPI = kLoaders / P_CPR;  // MC: chunks per k row, k rows per pass
+    constexpr int Q_CPR = BM / CE, Q_KPI = kLoaders / Q_CPR;
+    constexpr int kPassBytes = kLoaders * 16;  // LDS bytes filled by one 16-byte load of every loading thread
     constexpr int kPBufs = 3;
     constexpr int Q_BASE = kPBufs * P_BYTES;
 
-    // Slot q = it*kThreads + t of a slab is filled by thread t in pass it, so a wave fills
+    // Slot q = it*kLoaders + t of a slab is filled by thread t < kLoaders in pass it, so a wave fills
     // 1 KiB of consecutive LDS per load.  The swizzle is applied on the memory side: the
     // thread fetches the chunk that belongs in its slot.
     //   KC: slot q is row q/8, position q%8, and holds chunk (q%8) ^ swz(row)
@@ -375,11 +386,13 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             }
         }
     };
-    // adds up the chunks this thread's loads put into Q buffer `buf` (after they have landed)
+    // adds up this thread's share of the chunks in Q buffer `buf` (after they have landed):
+    // slots t, t + kThreads, ... -- the same column chunk in every one of them
+    constexpr int kBiasPasses = BM * 8 / kThreads, kBiasKPI = kThreads / Q_CPR;
     auto add_q_chunks = [&](int buf) {
         const unsigned char *sq = smem + Q_BASE + buf * Q_BYTES + t * 16;
 #pragma unroll
-        for (int it = 0; it < NQ; ++it) add_chunk(*(const u32x4 *)(sq + it * kPassBytes));
+        for (int it = 0; it < kBiasPasses; ++it) add_chunk(*(const u32x4 *)(sq + it * kThreads * 16));
     };
 
     // -- fragments ---------------------------------------------------------------
@@ -440,14 +453,24 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int kQReads = TJ * ((QSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1);
     constexpr int kReads = kPReads + kQReads;                   // LDS read instructions per step
     constexpr int kMfma = TI * TJ * (sizeof(T) == 4 ? 4 : 1);   // MFMA instructions per step
+#ifndef FMOE_X_RPM
+#define FMOE_X_RPM 2
+#endif
+#ifndef FMOE_X_SPLIT
+#define FMOE_X_SPLIT 1
+#endif
+    constexpr int kReadsPerMfma = FMOE_X_RPM;  // a step's reads go out early, the remaining MFMAs follow
+    constexpr int kSplit = FMOE_X_SPLIT;       // MFMA columns of the last step issued before the barrier
+    constexpr int kLoadsPerMfma = (NP + kMfma - 1) / kMfma;
 
     const int n_slabs = (K + BKE - 1) / BKE;
     u32x4 pf[2][TI], qf[2][TJ];
     auto read_step = [&](int buf, const unsigned char *sp, const unsigned char *sq, int ks) {
-#pragma unroll
-        for (int x = 0; x < TI; ++x) pf[buf][x] = frag(sp, PSHAPE, BN, wave_n0 + x * 32, ks);
+        // in the order the MFMAs (x outer, y inner) first need them
 #pragma unroll
         for (int y = 0; y < TJ; ++y) qf[buf][y] = frag(sq, QSHAPE, BM, wave_m0 + y * 32, ks);
+#pragma unroll
+        for (int x = 0; x < TI; ++x) pf[buf][x] = frag(sp, PSHAPE, BN, wave_n0 + x * 32, ks);
     };
     // s_waitcnt vmcnt(n) lgkmcnt(0): at most n of this wave's loads still in flight, all LDS reads done
     auto wait_loads = [&](auto n_tag) {
@@ -463,19 +486,27 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    auto main_loop = [&](auto with_bias) {
+    auto main_loop = [&](auto with_bias, auto loads_tag) {
         constexpr bool kBias = decltype(with_bias)::value;
-        issue_p(0, 0);
-        issue_q(0, 0);
-        issue_p(BKE, 1);
-        issue_q(BKE, 1);
+        constexpr bool kLoads = decltype(loads_tag)::value;  // this wave requests slabs
+        constexpr int kNoWait = 63;
+        if constexpr (kLoads) {
+            issue_p(0, 0);
+            issue_q(0, 0);
+            issue_p(BKE, 1);
+            issue_q(BKE, 1);
+        }
         __builtin_amdgcn_sched_barrier(0);
-        wait_loads(std::integral_constant<int, NP + NQ>{});  // slab 0 has landed
+        wait_loads(std::integral_constant<int, kLoads ? NP + NQ : kNoWait>{});  // slab 0 has landed
         slab_barrier();
         if constexpr (kBias) add_q_chunks(0);
         read_step(0, smem, smem + Q_BASE, 0);
         __builtin_amdgcn_sched_barrier(0);
 
+#ifdef FMOE_X_TIMING
+        unsigned long long dbg_compute = 0, dbg_wait = 0, dbg_bar = 0, dbg_last = __builtin_amdgcn_s_memtime();
+        const unsigned long long dbg_start = dbg_last;
+#endif
         int pc = 0;
         for (int s = 0; s < n_slabs; ++s) {
             const int pn = pc == kPBufs - 1 ? 0 : pc + 1;
@@ -484,7 +515,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             const unsigned char *sq = smem + Q_BASE + (s & 1) * Q_BYTES;
 #pragma unroll
             for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
-                if (ks == 0) issue_p((s + 2) * BKE, pf_buf);
+                if (kLoads && ks == 0) issue_p((s + 2) * BKE, pf_buf);
                 read_step((ks + 1) & 1, sp, sq, ks + 1);
 #pragma unroll
                 for (int x = 0; x < TI; ++x)
@@ -492,32 +523,47 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                     for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
 #pragma unroll
                 for (int i = 0; i < kMfma; ++i) {
-                    if (i < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one MFMA
-                    if (ks == 0 && i < NP) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
+                    if (i * kReadsPerMfma < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);  // LDS reads
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            // one MFMA
+                    if (kLoads && ks == 0 && i * kLoadsPerMfma < NP) __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPerMfma, 0);                     // one load
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
             constexpr int kLast = (kStepsPerSlab - 1) & 1;
 #pragma unroll
-            for (int x = 0; x < TI / 2; ++x)
+            for (int x = 0; x < kSplit; ++x)
 #pragma unroll
                 for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
             __builtin_amdgcn_sched_barrier(0);
-            wait_loads(std::integral_constant<int, NP>{});  // everything but the P loads of slab s+2
+#ifdef FMOE_X_TIMING
+            const unsigned long long tb = __builtin_amdgcn_s_memtime();
+            __builtin_amdgcn_sched_barrier(0);
+#endif
+            wait_loads(std::integral_constant<int, kLoads ? NP : kNoWait>{});  // everything but the P loads of slab s+2
+#ifdef FMOE_X_TIMING
+            __builtin_amdgcn_sched_barrier(0);
+            const unsigned long long tc = __builtin_amdgcn_s_memtime();
+#endif
             slab_barrier();
+#ifdef FMOE_X_TIMING
+            const unsigned long long td = __builtin_amdgcn_s_memtime();
+            dbg_compute += tb - dbg_last; dbg_wait += tc - tb; dbg_bar += td - tc; dbg_last = td;
+            __builtin_amdgcn_sched_barrier(0);
+#endif
             if constexpr (kBias) add_q_chunks((s + 1) & 1);
-            issue_q((s + 2) * BKE, s & 1);
+            if constexpr (kLoads) issue_q((s + 2) * BKE, s & 1);
             read_step(0, smem + pn * P_BYTES, smem + Q_BASE + ((s + 1) & 1) * Q_BYTES, 0);
 #pragma unroll
-            for (int x = TI / 2; x < TI; ++x)
+            for (int x = kSplit; x < TI; ++x)
 #pragma unroll
                 for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+            constexpr int kAfter = kMfma - kSplit * (kMfma / TI);  // MFMAs after the barrier
+            constexpr int kQLoadsPerMfma = (NQ + kAfter - 1) / kAfter;
 #pragma unroll
-            for (int i = 0; i < kMfma / 2; ++i) {
+            for (int i = 0; i < kAfter; ++i) {
+                if (i * kReadsPerMfma < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, (NQ + kMfma / 2 - 1) / (kMfma / 2), 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma / 2 - 1) / (kMfma / 2), 0);
+                if (kLoads && i * kQLoadsPerMfma < NQ) __builtin_amdgcn_sched_group_barrier(0x020, kQLoadsPerMfma, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
             pc = pn;
@@ -525,20 +571,31 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         // the loads requested past the last slab (all out of range) must land before LDS is reused
         wait_loads(std::integral_constant<int, 0>{});
         slab_barrier();
+#ifdef FMOE_X_TIMING
+        if (lane == 0 && blockIdx.x < 16384) {
+            unsigned long long *o = fmoe_dbg + (size_t)blockIdx.x * 8;
+            if (wave == 0) { o[0] = dbg_compute; o[1] = dbg_wait; o[2] = dbg_bar; o[3] = dbg_last - dbg_start; o[4] = dbg_start; }
+            if (wave == 7) { o[5] = dbg_compute; o[6] = dbg_wait; o[7] = dbg_bar; }
+        }
+#endif
+    };
+    auto run_loop = [&](auto with_bias) {
+        if (kLoadWaves == kWavesM * kWavesN || wave_u < (uint32_t)kLoadWaves) main_loop(with_bias, std::true_type{});
+        else main_loop(with_bias, std::false_type{});
     };
     bool want_bias = false;
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) want_bias = prm.bias_grad != nullptr && nt == 0;
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
-        if (want_bias) main_loop(std::true_type{});
-        else main_loop(std::false_type{});
+        if (want_bias) run_loop(std::true_type{});
+        else run_loop(std::false_type{});
     } else {
-        main_loop(std::false_type{});
+        run_loop(std::false_type{});
     }
 
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
         if (want_bias) {
-            // thread t holds CE columns of contraction rows t / Q_CPR (mod Q_KPI);
-            // the Q_KPI partial sums of a column are added in ascending order
+            // thread t holds CE columns of contraction rows t / Q_CPR (mod kBiasKPI);
+            // the kBiasKPI partial sums of a column are added in ascending order
             float *red = (float *)smem;
             __syncthreads();
             // the chunk this thread stages is the one that belongs in its (swizzled) slot
@@ -549,7 +606,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             if (t < BM && t < q_valid) {
                 float sum = 0.f;
 #pragma unroll
-                for (int g = 0; g < Q_KPI; ++g) sum += red[g * BM + t];
+                for (int g = 0; g < kBiasKPI; ++g) sum += red[g * BM + t];
                 T *dst = (T *)prm.bias_grad + (int64_t)expert * prm.n_rows + mt * BM + t;
                 if (prm.accumulate_first && ei == 0) sum += (float)*dst;
                 *dst = (T)sum;
