@@ -39,9 +39,3 @@ int FMOE_CAT(FMOE_TNAME, wgrad)(GemmParams &prm, int epilogue, hipStream_t strea
 #endif
 
 }  // namespace fmoe
-
-#ifdef FMOE_X_TIMING
-extern "C" int fmoe_x_dbg_read(unsigned long long *host, int n) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fmoe::gemm::fmoe_dbg), (size_t)n * 8);
-}
-#endif

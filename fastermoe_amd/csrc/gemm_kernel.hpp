@@ -18,26 +18,18 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Waves of a workgroup along C's rows and columns.  4 x 2 (512 threads, two waves per
-// SIMD, 64 x 128 per wave) keeps the matrix pipe fed while one wave sits at the
-// barrier or waits for LDS; 2 x 2 (256 threads, 128 x 128 per wave) halves the LDS
-// reads per MFMA.  FMOE_GEMM_WAVES_M selects at build time.
-#ifndef FMOE_GEMM_WAVES_M
-#define FMOE_GEMM_WAVES_M 4
-#endif
-constexpr int kWavesM = FMOE_GEMM_WAVES_M, kWavesN = 2;
+// Waves of a workgroup along C's rows and columns: 4 x 2 (512 threads, two waves per SIMD,
+// 64 x 128 per wave), so that the matrix pipe stays fed while one wave of a SIMD sits at
+// the barrier or waits for LDS.
+constexpr int kWavesM = 4, kWavesN = 2;
 constexpr int kThreads = 64 * kWavesM * kWavesN;
 // The first kLoadWaves waves of a workgroup request the slabs.  The SIMD issues from its
 // oldest wave first, so with two waves per SIMD the younger one falls behind; leaving the
 // loads (which can block at a full load queue) to the older waves evens the two out.
-#ifndef FMOE_X_LOADWAVES
-#define FMOE_X_LOADWAVES 4
-#endif
-constexpr int kLoadWaves = FMOE_X_LOADWAVES;
+constexpr int kLoadWaves = 4;
 constexpr int kLoaders = 64 * kLoadWaves;
 constexpr int kRowsPerPass = kLoaders / 8;  // KC slabs: rows covered by one 16-byte load of every loading thread
 constexpr int kSlabBytes = 128;  // contraction bytes per row per slab
-constexpr int kStepsPerSlab = 4; // 32-byte contraction steps (two 16-byte chunks) per slab
 constexpr int kGroupM = 8;       // row tiles that share a column tile consecutively
 
 enum Shape { kKC = 0, kMC = 1 };
@@ -46,10 +38,15 @@ enum Ragged { kRaggedRows = 0, kRaggedK = 1 };
 // ---- element traits ---------------------------------------------------------
 template <typename T> struct Elem;
 
+// The 16-bit types use the 16 x 16 x 32 MFMA (4 accumulator registers per block): for the same
+// flops it moves half as many accumulator registers as 32 x 32 x 16, and under the chip's
+// power limit that buys clock.  fp32 uses 32 x 32 x 2.
 template <> struct Elem<__bf16> {
     static constexpr int kPerChunk = 8;
-    __device__ static __forceinline__ void mma(f32x16 &acc, const u32x4 &p, const u32x4 &q) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, p), __builtin_bit_cast(bf16x8, q),
+    static constexpr int kBlk = 16;  // rows and columns of one MFMA block
+    typedef f32x4 Acc;
+    __device__ static __forceinline__ void mma(Acc &acc, const u32x4 &p, const u32x4 &q) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, p), __builtin_bit_cast(bf16x8, q),
                                                       acc, 0, 0, 0);
     }
     __device__ static __forceinline__ float to_float(__bf16 v) { return (float)v; }
@@ -57,15 +54,19 @@ template <> struct Elem<__bf16> {
 
 template <> struct Elem<_Float16> {
     static constexpr int kPerChunk = 8;
-    __device__ static __forceinline__ void mma(f32x16 &acc, const u32x4 &p, const u32x4 &q) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, p), __builtin_bit_cast(f16x8, q), acc,
+    static constexpr int kBlk = 16;
+    typedef f32x4 Acc;
+    __device__ static __forceinline__ void mma(Acc &acc, const u32x4 &p, const u32x4 &q) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, p), __builtin_bit_cast(f16x8, q), acc,
                                                      0, 0, 0);
     }
 };
 
 template <> struct Elem<float> {
     static constexpr int kPerChunk = 4;
-    __device__ static __forceinline__ void mma(f32x16 &acc, const u32x4 &p, const u32x4 &q) {
+    static constexpr int kBlk = 32;
+    typedef f32x16 Acc;
+    __device__ static __forceinline__ void mma(Acc &acc, const u32x4 &p, const u32x4 &q) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(p[j]), __uint_as_float(q[j]), acc, 0, 0, 0);
@@ -131,15 +132,15 @@ struct GemmParams {
 
 // KC slabs: 16-byte chunk c of row r is stored at chunk c ^ swz(r).
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
-// MC slabs of 16-bit elements: chunk c of contraction row k is stored at c ^ ((k % 4) * 4).
-// A transposing read of 32 lanes touches 4 k rows x 4 chunks (two 16-column blocks); rows
-// are a multiple of 256 B apart, so without the swizzle they would share banks -- with it
-// the 16 chunks fall on the 16 distinct 16-byte positions of the 256-byte bank cycle.
-template <typename T> __device__ __forceinline__ int mc_swz(int k) { return sizeof(T) == 2 ? (k & 3) << 2 : 0; }
+// MC slabs of 16-bit elements: chunk c of contraction row k is stored at
+// c ^ ((k % 4) * 4 + (k / 8 % 2) * 2).  A transposing read of 32 lanes touches two blocks of
+// 4 k rows x 2 chunks, 8 k rows apart; rows are a multiple of 256 B apart, so without the
+// swizzle they would share banks -- with it the 16 chunks fall on the 16 distinct 16-byte
+// positions of the 256-byte bank cycle.
+template <typename T> __device__ __forceinline__ int mc_swz(int k) {
+    return sizeof(T) == 2 ? ((k & 3) << 2) | (((k >> 3) & 1) << 1) : 0;
+}
 
-#ifdef FMOE_X_TIMING
-__device__ unsigned long long fmoe_dbg[8 * 16384];
-#endif
 // ---- the kernel ---------------------------------------------------------------
 template <typename T, int BM, int BN, int PSHAPE, int QSHAPE, int RAGGED, int EPI>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
@@ -147,7 +148,10 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int CE = Elem<T>::kPerChunk;           // elements per 16-byte chunk
     constexpr int BKE = kSlabBytes / (int)sizeof(T); // elements per slab row
     constexpr int WM = BM / kWavesM, WN = BN / kWavesN;  // wave tile
-    constexpr int TI = WN / 32, TJ = WM / 32;        // MFMA blocks per wave (cols, rows)
+    constexpr int MB = Elem<T>::kBlk;                // MFMA block edge
+    constexpr int TI = WN / MB, TJ = WM / MB;        // MFMA blocks per wave (cols, rows)
+    constexpr int kAccRegs = MB * MB / 64;           // accumulator registers per block
+    constexpr int kChunksPerStep = 64 / MB;          // 16-byte contraction chunks one MFMA step consumes per row
     constexpr int NP = BN * 8 / kLoaders;            // 16-byte chunks per loading thread per slab
     constexpr int NQ = BM * 8 / kLoaders;
     constexpr int P_BYTES = BN * kSlabBytes, Q_BYTES = BM * kSlabBytes;
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
-    const int l32 = lane & 31, h = lane >> 5;
+    const int lb = lane & (MB - 1), hq = lane / MB;  // row inside an MFMA block, contraction chunk inside a step
     const int wave_m0 = (wave / kWavesN) * WM, wave_n0 = (wave % kWavesN) * WN;
 
     // An expert without rows has a zero weight gradient (and bias gradient): write the
@@ -277,12 +281,14 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                              ? (uint32_t)(((int64_t)(it * kRowsPerPass + r) * prm.ldp + p_kc_chunk * CE) * sizeof(T))
                              : kOutOfRange;
     } else {
-        const int kk = t / P_CPR, c = (t % P_CPR) ^ mc_swz<T>(kk);
+        const int kk = t / P_CPR;
 #pragma unroll
-        for (int it = 0; it < NP; ++it)
+        for (int it = 0; it < NP; ++it) {
+            const int c = (t % P_CPR) ^ mc_swz<T>(it * P_KPI + kk);
             p_voff[it] = (c * CE < p_valid)
                              ? (uint32_t)(((int64_t)(it * P_KPI + kk) * prm.ldp + c * CE) * sizeof(T))
                              : kOutOfRange;
+        }
     }
     if (QSHAPE == kKC) {
         const int r = t >> 3;
@@ -293,12 +299,14 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                              ? (uint32_t)(((int64_t)(it * kRowsPerPass + r) * prm.ldq + q_kc_chunk * CE) * sizeof(T))
                              : kOutOfRange;
     } else {
-        const int kk = t / Q_CPR, c = (t % Q_CPR) ^ mc_swz<T>(kk);
+        const int kk = t / Q_CPR;
 #pragma unroll
-        for (int it = 0; it < NQ; ++it)
+        for (int it = 0; it < NQ; ++it) {
+            const int c = (t % Q_CPR) ^ mc_swz<T>(it * Q_KPI + kk);
             q_voff[it] = (c * CE < q_valid)
                              ? (uint32_t)(((int64_t)(it * Q_KPI + kk) * prm.ldq + c * CE) * sizeof(T))
                              : kOutOfRange;
+        }
     }
 
     // With an MC slab the fragments are read by ds_read_b64_tr_b16, and the compiler puts a
@@ -396,29 +404,31 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     };
 
     // -- fragments ---------------------------------------------------------------
-    // A fragment is the 16 bytes a lane feeds to the MFMA for one 32-row block and
-    // one contraction step: row = block row l32, contraction chunk = 2*step + h.
+    // A fragment is the 16 bytes a lane feeds to the MFMA for one block of MB rows and one
+    // contraction step (64 bytes of the slab row for 16-bit types, 32 for fp32):
+    // row = block row lb, contraction chunk = kChunksPerStep * step + hq.
     auto frag = [&](const unsigned char *slab, int shape, int extent, int r0, int ks) -> u32x4 {
-        const int row = r0 + l32;
         if (shape == kKC) {
-            const int chunk = ks * 2 + h;
+            const int row = r0 + lb;
+            const int chunk = ks * kChunksPerStep + hq;
             return *(const u32x4 *)(slab + row * kSlabBytes + ((chunk ^ swz(row)) << 4));
         }
         u32x4 out;
-        if (sizeof(T) == 4) {
+        if constexpr (sizeof(T) == 4) {
+            const int row = r0 + lb;
             const uint32_t *s = (const uint32_t *)slab;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) out[j] = s[(ks * 8 + h * 4 + j) * extent + row];
+            for (int j = 0; j < 4; ++j) out[j] = s[(ks * 8 + hq * 4 + j) * extent + row];
         } else {
             // ds_read_b64_tr_b16: a 16-lane group reads a 4(k) x 16(row) block of 16-bit
             // elements, lane s of the group pointing at row-of-k s/4, columns 4*(s%4)..+3,
-            // and receives column s of the block with its 4 k values.  Groups 0/1 take rows
-            // 0-15/16-31 of the 32-row block, groups 2/3 the same rows 8 k further on.
-            const int grp = lane >> 4, s16 = lane & 15;
-            const int col = r0 + (grp & 1) * 16 + 4 * (s16 & 3);
-            const int kq = s16 >> 2;
-            const int chunk = (col >> 3) ^ (kq << 2);   // MC slabs are swizzled by k % 4
-            const int kb = ks * 16 + (grp >> 1) * 8 + kq;
+            // and receives column s of the block with its 4 k values.  Group g takes the 16
+            // rows of the MFMA block at contraction indices 8g..8g+3 of the step; the
+            // second read is 4 k further on.
+            const int s16 = lane & 15;
+            const int col = r0 + 4 * (s16 & 3);
+            const int kb = ks * 32 + hq * 8 + (s16 >> 2);
+            const int chunk = (col >> 3) ^ mc_swz<T>(kb);  // kb and kb + 4 swizzle alike
             const unsigned char *base = slab + chunk * 16 + (col & 7) * 2;
             typedef short s16x4 __attribute__((ext_vector_type(4)));
             typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_ptr;
@@ -430,47 +440,61 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         return out;
     };
 
-    f32x16 acc[TI][TJ];
+    typename Elem<T>::Acc acc[TI][TJ];
 #pragma unroll
     for (int x = 0; x < TI; ++x)
 #pragma unroll
         for (int y = 0; y < TJ; ++y)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[x][y][r] = 0.f;
+            for (int r = 0; r < kAccRegs; ++r) acc[x][y][r] = 0.f;
 
-    // Main loop, one basic block per slab, software-pipelined by hand.  P buffer pc holds
-    // slab s, pn slab s+1, pf receives slab s+2; Q buffer s%2 holds slab s.  Per slab:
-    //   step 0     : MFMAs of step 0, LDS reads of step 1, and the P loads of slab s+2
-    //   steps 1..2 : MFMAs of step ks, LDS reads of step ks+1 between them
-    //   step 3a    : first half of the last step's MFMAs, then wait until this wave's loads
-    //                of slab s+1 have landed (the P loads of slab s+2 stay in flight)
-    //   barrier    : slab s+1 is complete and nobody reads slab s any more
-    //   step 3b    : second half of the MFMAs; the Q part of slab s+2 is requested into the
-    //                Q buffer of slab s and step 0 of slab s+1 is read
+    // Main loop, one basic block per slab, software-pipelined by hand.  A slab is worked
+    // through in four phases.  fp32 (32 x 32 blocks): a phase is one contraction step over
+    // all block columns.  16-bit (16 x 16 blocks): a phase is half the block columns of one
+    // of the slab's two contraction steps, so the Q fragments are read every other phase.
+    // P buffer pc holds slab s, pn slab s+1, pf_buf receives slab s+2; Q buffer s%2 holds
+    // slab s.  Per slab:
+    //   phase 0     : MFMAs of phase 0, LDS reads of phase 1, and the P loads of slab s+2
+    //   phases 1..2 : MFMAs of the phase, LDS reads of the next one between them
+    //   phase 3a    : the first MFMAs of the last phase, then wait until this wave's loads
+    //                 of slab s+1 have landed (the P loads of slab s+2 stay in flight)
+    //   barrier     : slab s+1 is complete and nobody reads slab s any more
+    //   phase 3b    : the rest of the MFMAs; the Q part of slab s+2 is requested into the
+    //                 Q buffer of slab s and phase 0 of slab s+1 is read
     // so no LDS read is waited for at the top of an iteration.  Past the last slab the
     // loads return zeros and land in buffers nobody reads, which keeps the body branch-free.
-    constexpr int kPReads = TI * ((PSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1);
-    constexpr int kQReads = TJ * ((QSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1);
-    constexpr int kReads = kPReads + kQReads;                   // LDS read instructions per step
-    constexpr int kMfma = TI * TJ * (sizeof(T) == 4 ? 4 : 1);   // MFMA instructions per step
-#ifndef FMOE_X_RPM
-#define FMOE_X_RPM 2
-#endif
-#ifndef FMOE_X_SPLIT
-#define FMOE_X_SPLIT 1
-#endif
-    constexpr int kReadsPerMfma = FMOE_X_RPM;  // a step's reads go out early, the remaining MFMAs follow
-    constexpr int kSplit = FMOE_X_SPLIT;       // MFMA columns of the last step issued before the barrier
+    constexpr int kPhases = 4;
+    constexpr int PF = (MB == 32) ? TI : TI / 2;                // block columns per phase
+    constexpr int kPReadsPerFrag = (PSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1;
+    constexpr int kQReadsPerFrag = (QSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1;
+    constexpr int kMfma = PF * TJ * (sizeof(T) == 4 ? 4 : 1);   // MFMA instructions per phase
+    constexpr int kMfmaPerCol = kMfma / PF;
+    constexpr int kReadsPerMfma = 1;  // a phase's reads go out early, one per MFMA; the remaining MFMAs follow
+    constexpr int kSplit = 1;         // block columns of the last phase issued before the barrier
     constexpr int kLoadsPerMfma = (NP + kMfma - 1) / kMfma;
+    // contraction step, first block column, Q fragment buffer of a phase; does it start a step
+    auto phase_ks = [](int ph) { return MB == 32 ? ph : ph >> 1; };
+    auto phase_x0 = [](int ph) { return MB == 32 ? 0 : (ph & 1) * PF; };
+    auto phase_qbuf = [](int ph) { return MB == 32 ? (ph & 1) : ((ph >> 1) & 1); };
+    auto phase_reads_q = [](int ph) { return MB == 32 || (ph & 1) == 0; };
+    auto phase_reads = [&](int ph) { return PF * kPReadsPerFrag + (phase_reads_q(ph) ? TJ * kQReadsPerFrag : 0); };
 
     const int n_slabs = (K + BKE - 1) / BKE;
-    u32x4 pf[2][TI], qf[2][TJ];
-    auto read_step = [&](int buf, const unsigned char *sp, const unsigned char *sq, int ks) {
-        // in the order the MFMAs (x outer, y inner) first need them
+    u32x4 pf[2][PF], qf[2][TJ];
+    // the fragments of phase ph, in the order its MFMAs (x outer, y inner) first need them
+    auto read_phase = [&](int ph, const unsigned char *sp, const unsigned char *sq) {
+        if (phase_reads_q(ph)) {
 #pragma unroll
-        for (int y = 0; y < TJ; ++y) qf[buf][y] = frag(sq, QSHAPE, BM, wave_m0 + y * 32, ks);
+            for (int y = 0; y < TJ; ++y) qf[phase_qbuf(ph)][y] = frag(sq, QSHAPE, BM, wave_m0 + y * MB, phase_ks(ph));
+        }
 #pragma unroll
-        for (int x = 0; x < TI; ++x) pf[buf][x] = frag(sp, PSHAPE, BN, wave_n0 + x * 32, ks);
+        for (int x = 0; x < PF; ++x) pf[ph & 1][x] = frag(sp, PSHAPE, BN, wave_n0 + (phase_x0(ph) + x) * MB, phase_ks(ph));
+    };
+    auto mma_phase = [&](int ph, int x_lo, int x_hi) {
+#pragma unroll
+        for (int x = x_lo; x < x_hi; ++x)
+#pragma unroll
+            for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[phase_x0(ph) + x][y], pf[ph & 1][x], qf[phase_qbuf(ph)][y]);
     };
     // s_waitcnt vmcnt(n) lgkmcnt(0): at most n of this wave's loads still in flight, all LDS reads done
     auto wait_loads = [&](auto n_tag) {
@@ -500,13 +524,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         wait_loads(std::integral_constant<int, kLoads ? NP + NQ : kNoWait>{});  // slab 0 has landed
         slab_barrier();
         if constexpr (kBias) add_q_chunks(0);
-        read_step(0, smem, smem + Q_BASE, 0);
+        read_phase(0, smem, smem + Q_BASE);
         __builtin_amdgcn_sched_barrier(0);
 
-#ifdef FMOE_X_TIMING
-        unsigned long long dbg_compute = 0, dbg_wait = 0, dbg_bar = 0, dbg_last = __builtin_amdgcn_s_memtime();
-        const unsigned long long dbg_start = dbg_last;
-#endif
         int pc = 0;
         for (int s = 0; s < n_slabs; ++s) {
             const int pn = pc == kPBufs - 1 ? 0 : pc + 1;
@@ -514,54 +534,31 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             const unsigned char *sp = smem + pc * P_BYTES;
             const unsigned char *sq = smem + Q_BASE + (s & 1) * Q_BYTES;
 #pragma unroll
-            for (int ks = 0; ks + 1 < kStepsPerSlab; ++ks) {
-                if (kLoads && ks == 0) issue_p((s + 2) * BKE, pf_buf);
-                read_step((ks + 1) & 1, sp, sq, ks + 1);
-#pragma unroll
-                for (int x = 0; x < TI; ++x)
-#pragma unroll
-                    for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[ks & 1][x], qf[ks & 1][y]);
+            for (int ph = 0; ph + 1 < kPhases; ++ph) {
+                if (kLoads && ph == 0) issue_p((s + 2) * BKE, pf_buf);
+                read_phase(ph + 1, sp, sq);
+                mma_phase(ph, 0, PF);
 #pragma unroll
                 for (int i = 0; i < kMfma; ++i) {
-                    if (i * kReadsPerMfma < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);  // LDS reads
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            // one MFMA
-                    if (kLoads && ks == 0 && i * kLoadsPerMfma < NP) __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPerMfma, 0);                     // one load
+                    if (i * kReadsPerMfma < phase_reads(ph + 1)) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);  // LDS reads
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       // one MFMA
+                    if (kLoads && ph == 0 && i * kLoadsPerMfma < NP) __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPerMfma, 0);  // loads
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            constexpr int kLast = (kStepsPerSlab - 1) & 1;
-#pragma unroll
-            for (int x = 0; x < kSplit; ++x)
-#pragma unroll
-                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
+            mma_phase(kPhases - 1, 0, kSplit);
             __builtin_amdgcn_sched_barrier(0);
-#ifdef FMOE_X_TIMING
-            const unsigned long long tb = __builtin_amdgcn_s_memtime();
-            __builtin_amdgcn_sched_barrier(0);
-#endif
             wait_loads(std::integral_constant<int, kLoads ? NP : kNoWait>{});  // everything but the P loads of slab s+2
-#ifdef FMOE_X_TIMING
-            __builtin_amdgcn_sched_barrier(0);
-            const unsigned long long tc = __builtin_amdgcn_s_memtime();
-#endif
             slab_barrier();
-#ifdef FMOE_X_TIMING
-            const unsigned long long td = __builtin_amdgcn_s_memtime();
-            dbg_compute += tb - dbg_last; dbg_wait += tc - tb; dbg_bar += td - tc; dbg_last = td;
-            __builtin_amdgcn_sched_barrier(0);
-#endif
             if constexpr (kBias) add_q_chunks((s + 1) & 1);
             if constexpr (kLoads) issue_q((s + 2) * BKE, s & 1);
-            read_step(0, smem + pn * P_BYTES, smem + Q_BASE + ((s + 1) & 1) * Q_BYTES, 0);
-#pragma unroll
-            for (int x = kSplit; x < TI; ++x)
-#pragma unroll
-                for (int y = 0; y < TJ; ++y) Elem<T>::mma(acc[x][y], pf[kLast][x], qf[kLast][y]);
-            constexpr int kAfter = kMfma - kSplit * (kMfma / TI);  // MFMAs after the barrier
+            read_phase(0, smem + pn * P_BYTES, smem + Q_BASE + ((s + 1) & 1) * Q_BYTES);
+            mma_phase(kPhases - 1, kSplit, PF);
+            constexpr int kAfter = kMfma - kSplit * kMfmaPerCol;  // MFMAs after the barrier
             constexpr int kQLoadsPerMfma = (NQ + kAfter - 1) / kAfter;
 #pragma unroll
             for (int i = 0; i < kAfter; ++i) {
-                if (i * kReadsPerMfma < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);
+                if (i * kReadsPerMfma < phase_reads(0)) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if (kLoads && i * kQLoadsPerMfma < NQ) __builtin_amdgcn_sched_group_barrier(0x020, kQLoadsPerMfma, 0);
             }
@@ -571,16 +568,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         // the loads requested past the last slab (all out of range) must land before LDS is reused
         wait_loads(std::integral_constant<int, 0>{});
         slab_barrier();
-#ifdef FMOE_X_TIMING
-        if (lane == 0 && blockIdx.x < 16384) {
-            unsigned long long *o = fmoe_dbg + (size_t)blockIdx.x * 8;
-            if (wave == 0) { o[0] = dbg_compute; o[1] = dbg_wait; o[2] = dbg_bar; o[3] = dbg_last - dbg_start; o[4] = dbg_start; }
-            if (wave == 7) { o[5] = dbg_compute; o[6] = dbg_wait; o[7] = dbg_bar; }
-        }
-#endif
     };
     auto run_loop = [&](auto with_bias) {
-        if (kLoadWaves == kWavesM * kWavesN || wave_u < (uint32_t)kLoadWaves) main_loop(with_bias, std::true_type{});
+        if (wave_u < (uint32_t)kLoadWaves) main_loop(with_bias, std::true_type{});
         else main_loop(with_bias, std::false_type{});
     };
     bool want_bias = false;
@@ -615,9 +605,10 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     }
 
     // -- epilogue ------------------------------------------------------------------
-    // acc[x][y][4*g + i] is C(row = wave_m0 + 32*y + l32, col = wave_n0 + 32*x + 8*g + 4*h + i):
-    // a lane owns 4 consecutive columns of 32 different rows, which written straight to
-    // memory would touch 32 cache lines per store.  Instead every wave passes its sub-tile
+    // acc[x][y][4*g + i] is C(row = wave_m0 + MB*y + lb, col = wave_n0 + MB*x + 8*g + 4*hq + i)
+    // (32 x 32 blocks: g = 0..3, hq = 0..1; 16 x 16 blocks: g = 0, hq = 0..3): a lane owns
+    // runs of 4 consecutive columns in many different rows, which written straight to
+    // memory would touch one cache line per row and store.  Instead every wave passes its sub-tile
     // through a private LDS staging area of [WM rows][256 B + 16 B pad] and moves it
     // between LDS and memory with 16-byte accesses that cover whole 256-byte row pieces
     // (4 rows per wave instruction).  Tiles that are read in the epilogue (the saved
@@ -627,7 +618,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     }
     constexpr int kStgRow = 256 + 16;            // bytes; the pad spreads rows over the banks
     constexpr int CPP = 256 / (int)sizeof(T);    // C columns per pass through the staging area
-    constexpr int XPP = CPP / 32;                // 32-column MFMA blocks per pass
+    constexpr int XPP = CPP / MB;                // MFMA block columns per pass
     constexpr int NPASS = WN / CPP;
     unsigned char *stg = smem + wave * (WM * kStgRow);
     const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride + n0 : nullptr;
@@ -693,8 +684,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             for (int xx = 0; xx < XPP; ++xx) {
                 const int x = pass * XPP + xx;
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int cip = xx * 32 + g * 8 + h * 4;  // column inside this pass
+                for (int g = 0; g < kAccRegs / 4; ++g) {
+                    const int cip = xx * MB + g * 8 + hq * 4;  // column inside this pass
                     float b4[4] = {0.f, 0.f, 0.f, 0.f};
                     if (bias && col_base + cip < p_valid) {
                         alignas(16) T bv[4];
@@ -705,7 +696,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                     }
 #pragma unroll
                     for (int y = 0; y < TJ; ++y) {
-                        const int row = y * 32 + l32;
+                        const int row = y * MB + lb;
                         float v[4];
 #pragma unroll
                         for (int i = 0; i < 4; ++i) v[i] = acc[x][y][4 * g + i] + b4[i];
