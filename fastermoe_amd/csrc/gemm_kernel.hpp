@@ -667,6 +667,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         for (int i = 0; i < 4; ++i) v[i] = (float)in[i];
     };
 
+    // The activation and the accumulate flag are fixed per launch; the epilogue is instantiated
+    // per value so that its element loop is straight-line code.
+    auto run_epilogue = [&](auto act_tag, auto accum_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
+    constexpr bool kAccum = decltype(accum_tag)::value;
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
         const int col_base = wave_n0 + pass * CPP;
@@ -675,7 +680,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
         for (int kind = kKinds - 1; kind >= 0; --kind) {
             if (EPI == kEpiBiasAct && kind == 1 && !aux) continue;
-            const bool reads_tile = (EPI == kEpiDAct) || accumulate;
+            constexpr bool reads_tile = (EPI == kEpiDAct) || kAccum;
             if (reads_tile) {
                 stage_in(EPI == kEpiDAct ? (const T *)aux : (const T *)Cb, col_base);
                 lds_sync();
@@ -702,14 +707,14 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                         for (int i = 0; i < 4; ++i) v[i] = acc[x][y][4 * g + i] + b4[i];
                         if (EPI == kEpiBiasAct && kind == 0) {
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) v[i] = apply_act(v[i], prm.activation);
+                            for (int i = 0; i < 4; ++i) v[i] = apply_act(v[i], ACT);
                         }
                         if (reads_tile) {
                             float in[4];
                             get4(row, cip, in);
 #pragma unroll
                             for (int i = 0; i < 4; ++i)
-                                v[i] = (EPI == kEpiDAct) ? v[i] * act_grad(in[i], prm.activation) : v[i] + in[i];
+                                v[i] = (EPI == kEpiDAct) ? v[i] * act_grad(in[i], ACT) : v[i] + in[i];
                         }
                         put4(row, cip, v);
                     }
@@ -719,6 +724,16 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             stage_out((EPI == kEpiBiasAct && kind == 1) ? aux : Cb, col_base);
             lds_sync();
         }
+    }
+    };
+    typedef std::integral_constant<int, FMOE_ACT_NONE> ActNone;
+    if constexpr (EPI == kEpiStore) {
+        if (accumulate) run_epilogue(ActNone{}, std::true_type{});
+        else run_epilogue(ActNone{}, std::false_type{});
+    } else {
+        if (prm.activation == FMOE_ACT_GELU) run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{});
+        else if (prm.activation == FMOE_ACT_RELU) run_epilogue(std::integral_constant<int, FMOE_ACT_RELU>{}, std::false_type{});
+        else run_epilogue(ActNone{}, std::false_type{});
     }
 #endif  // __HIP_DEVICE_COMPILE__
 }

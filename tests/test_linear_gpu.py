@@ -63,6 +63,42 @@ def test_linear_forward_backward(dtype, rows, e, fin, fout, bias, empties, devic
         assert gb is None
 
 
+# The grouped GEMM keeps three slabs of 128 contraction bytes in flight (64 bf16 / 32 fp32
+# elements each): contraction lengths of one to five slabs, with and without a ragged tail,
+# for the forward/data-grad (contraction = features) and the weight-grad (contraction = the
+# expert's rows), several row and column tiles per expert, and both tile heights (launches
+# of 512 tiles and more use 256-row tiles, smaller ones 128).
+DEPTH_CASES = [  # rows, experts, in, out
+    (300, 2, 64, 264),      # one slab (bf16), column tail
+    (520, 2, 128, 256),     # two slabs
+    (600, 3, 192, 520),     # three slabs: every P buffer used once
+    (700, 2, 200, 300),     # three slabs and a tail of 8
+    (1100, 2, 328, 272),    # five slabs and a tail, experts of 4-5 row tiles
+    (63, 1, 64, 256),       # weight-grad contraction shorter than a slab
+    (129, 2, 72, 8200),     # 33 column tiles
+    (9000, 2, 256, 4100),   # 36 x 17 tiles of 256 rows: the 256-row kernel with ragged tails
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,e,fin,fout", DEPTH_CASES)
+def test_linear_pipeline_depths(dtype, rows, e, fin, fout, device):
+    g = torch.Generator().manual_seed(rows * 7 + fin)
+    counts = ragged_counts(rows, e, g, 0)
+    x = torch.randn(rows, fin, generator=g).to(dtype)
+    w = (torch.randn(e, fout, fin, generator=g) / fin ** 0.5).to(dtype)
+    b = torch.randn(e, fout, generator=g).to(dtype)
+    gy = torch.randn(rows, fout, generator=g).to(dtype)
+    ref_y, ref_gx, ref_gw, ref_gb = _reference(x, counts, w, b, gy)
+    xd, wd, bd, gyd = x.to(device), w.to(device), b.to(device), gy.to(device)
+    tol = TOL[dtype]
+    assert rel_err(fmoe_native.linear_forward(xd, counts, wd, bd), ref_y) <= tol
+    gx, gw, gb = fmoe_native.linear_backward(gyd, xd, counts, wd, bd)
+    assert rel_err(gx, ref_gx) <= tol
+    assert rel_err(gw, ref_gw) <= tol
+    assert rel_err(gb, ref_gb) <= tol
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_moelinear_autograd(dtype, device):
     g = torch.Generator().manual_seed(1)
