@@ -47,6 +47,8 @@ SIGNATURES = {
                                        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
     "fmoe_combine_forward": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_combine_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "fmoe_gather_combine_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "fmoe_gather_combine_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "fmoe_profile_enable": (_int, [_int]),
     "fmoe_profile_classes": (_int, []),
     "fmoe_profile_collect": (_int, [_vp, _vp, _vp, _int]),

@@ -157,7 +157,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
         return rc;
     const int64_t n_slots = n_tokens * top_k;
     if (n_slots == 0) return FMOE_OK;
-    FMOE_REQUIRE(out && slot_to_row, "fmoe_fused_mlp_forward: NULL out / slot_to_row");
+    FMOE_REQUIRE(slot_to_row || !out, "fmoe_fused_mlp_forward: NULL slot_to_row");
     FMOE_REQUIRE(n_rows == 0 || (inp && pos && buf_in && buf_mid && buf_out),
                  "fmoe_fused_mlp_forward: NULL buffer");
     const int dt = p->dtype;
@@ -170,7 +170,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     chunk_bounds(expert_count_host, E, n_rows, n_chunks, bounds);
 
     // dropped slots become zero rows; independent of everything else
-    if (n_rows < n_slots)
+    if (out && n_rows < n_slots)
         if (int rc = permute_zero_unmapped(slot_to_row, out, n_slots, d, dt, l->out)) return rc;
 
     for (int c = 0; c < n_chunks; ++c) {
@@ -191,7 +191,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
         if (int rc = grouped_linear_forward(f2, expert_count_host, E, lo, hi, l->compute)) return rc;
         FMOE_HIP_CHECK(hipEventRecord(l->out_ready[c], l->compute));
     }
-    for (int c = 0; c < n_chunks; ++c) {
+    for (int c = 0; c < n_chunks && out; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         FMOE_HIP_CHECK(hipStreamWaitEvent(l->out, l->out_ready[c], 0));
@@ -212,7 +212,7 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
         return rc;
     FMOE_REQUIRE(grad_w1 && grad_w2, "fmoe_fused_mlp_backward: NULL weight gradient");
     FMOE_REQUIRE(n_tokens == 0 || (grad_inp && slot_to_row), "fmoe_fused_mlp_backward: NULL grad_inp / slot_to_row");
-    FMOE_REQUIRE(n_rows == 0 || (grad_out && pos && buf_in && buf_mid && g_out && g_mid && g_in),
+    FMOE_REQUIRE(n_rows == 0 || ((pos || !grad_out) && buf_in && buf_mid && g_out && g_mid && g_in),
                  "fmoe_fused_mlp_backward: NULL buffer");
     FMOE_REQUIRE(p->activation == FMOE_ACT_NONE || n_rows == 0 || buf_pre,
                  "fmoe_fused_mlp_backward: pre-activation buffer is NULL");
@@ -229,9 +229,10 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
-        // permute-in: g_out[r] = grad_out[pos[r]]
-        if (int rc = permute_gather_rows(grad_out, pos + lo, 1, at(g_out, lo, d, dt), hi - lo, n_slots, d, dt, l->in))
-            return rc;
+        // permute-in: g_out[r] = grad_out[pos[r]] (nothing to do when the caller filled g_out)
+        if (grad_out)
+            if (int rc = permute_gather_rows(grad_out, pos + lo, 1, at(g_out, lo, d, dt), hi - lo, n_slots, d, dt, l->in))
+                return rc;
         FMOE_HIP_CHECK(hipEventRecord(l->in_ready[c], l->in));
     }
     // The last chunk (even when it is empty) also zero-fills the experts without rows.

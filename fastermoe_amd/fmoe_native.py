@@ -226,6 +226,40 @@ def combine_backward(grad_out, x, score, n_tokens, top_k):
     return grad_x, grad_score
 
 
+def gather_combine_forward(rows, slot_to_row, score, n_tokens, top_k):
+    """out[t] = sum_j score[t,j] * rows[slot_to_row[t*top_k+j]] (dropped slots, index < 0,
+    contribute nothing): MOEGather's copy to slot order and the bmm in one pass."""
+    dt = _rows("rows", rows)
+    _dev("score", score, rows.dtype)
+    _dev("slot_to_row", slot_to_row, torch.int64)
+    if slot_to_row.numel() != n_tokens * top_k or score.numel() != n_tokens * top_k:
+        raise ValueError("slot_to_row and score must have n_tokens*top_k entries")
+    out = torch.empty(n_tokens, rows.shape[1], dtype=rows.dtype, device=rows.device)
+    with torch.cuda.device(rows.device):
+        check(_lib.load().fmoe_gather_combine_forward(_ptr(rows), _ptr(slot_to_row), _ptr(score), _ptr(out), n_tokens,
+                                                      top_k, rows.shape[0], rows.shape[1], dt, _stream(rows)))
+    return out
+
+
+def gather_combine_backward(grad_out, rows, slot_to_row, score, n_tokens, top_k):
+    """Returns (grad_rows [n_rows, d] in expert-sorted order, grad_score [N, top_k])."""
+    dt = _rows("rows", rows)
+    _dev("grad_out", grad_out, rows.dtype)
+    _dev("score", score, rows.dtype)
+    _dev("slot_to_row", slot_to_row, torch.int64)
+    if tuple(grad_out.shape) != (n_tokens, rows.shape[1]):
+        raise ValueError(f"grad_out must be [{n_tokens}, {rows.shape[1]}]")
+    if slot_to_row.numel() != n_tokens * top_k or score.numel() != n_tokens * top_k:
+        raise ValueError("slot_to_row and score must have n_tokens*top_k entries")
+    grad_rows = torch.empty_like(rows)
+    grad_score = torch.empty(n_tokens, top_k, dtype=rows.dtype, device=rows.device)
+    with torch.cuda.device(rows.device):
+        check(_lib.load().fmoe_gather_combine_backward(_ptr(grad_out), _ptr(rows), _ptr(slot_to_row), _ptr(score),
+                                                       _ptr(grad_rows), _ptr(grad_score), n_tokens, top_k,
+                                                       rows.shape[0], rows.shape[1], dt, _stream(rows)))
+    return grad_rows, grad_score
+
+
 # ---- per-expert linear ----------------------------------------------------------
 
 def _check_linear(input_buf, expert_count, weight, bias):
@@ -303,10 +337,13 @@ def _mlp_params(w1, b1, w2, b2, activation):
     return prm, n_expert, d_model, d_hidden
 
 
-def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k, activation, n_chunks):
+def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k, activation, n_chunks,
+                      slot_order=True):
     """scatter -> Linear -> activation -> Linear -> gather as one pipelined call.
     Returns ``(out [N*top_k, d], buf_in, buf_pre or None, buf_mid)``; the three
-    buffers are what the backward needs."""
+    buffers are what the backward needs.  With ``slot_order=False`` the copy to
+    slot order is skipped and ``out`` is the experts' output in expert-sorted
+    order, ``[n_rows, d]``."""
     prm, n_expert, d_model, d_hidden = _mlp_params(w1, b1, w2, b2, activation)
     _dev("inp", inp, w1.dtype)
     _dev("pos", pos, torch.int64)
@@ -320,38 +357,42 @@ def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k
     new = lambda r, c: torch.empty(r, c, dtype=inp.dtype, device=inp.device)
     buf_in, buf_mid, buf_out = new(n_rows, d_model), new(n_rows, d_hidden), new(n_rows, d_model)
     buf_pre = new(n_rows, d_hidden) if activation == _lib.ACT_GELU else None
-    out = new(n_tokens * top_k, d_model)
+    out = new(n_tokens * top_k, d_model) if slot_order else None
     with torch.cuda.device(inp.device):
         check(_lib.load().fmoe_fused_mlp_forward(
             ctypes.byref(prm), _ptr(inp), _ptr(pos), _ptr(slot_to_row), ctypes.c_void_p(cnt.data_ptr()),
             n_tokens, top_k, n_rows, _ptr(buf_in), _ptr(buf_pre), _ptr(buf_mid), _ptr(buf_out), _ptr(out),
             n_chunks, _stream(inp)))
-    return out, buf_in, buf_pre, buf_mid
+    return (out if slot_order else buf_out), buf_in, buf_pre, buf_mid
 
 
 def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid,
-                       n_tokens, top_k, activation, n_chunks):
+                       n_tokens, top_k, activation, n_chunks, slot_order=True):
     """Backward of :func:`fused_mlp_forward`.  Returns
     ``(grad_inp, grad_w1, grad_b1, grad_w2, grad_b2)`` (bias grads ``None``
     without biases).  For ReLU the post-activation buffer doubles as the
-    pre-activation (same sign pattern)."""
+    pre-activation (same sign pattern).  With ``slot_order=False``, ``grad_out``
+    is already in expert-sorted order, ``[n_rows, d]``."""
     prm, n_expert, d_model, d_hidden = _mlp_params(w1, b1, w2, b2, activation)
     _dev("grad_out", grad_out, w1.dtype)
-    if tuple(grad_out.shape) != (n_tokens * top_k, d_model):
-        raise ValueError(f"grad_out must be [{n_tokens * top_k}, {d_model}]")
     n_rows = pos.numel()
+    want = (n_tokens * top_k, d_model) if slot_order else (n_rows, d_model)
+    if tuple(grad_out.shape) != want:
+        raise ValueError(f"grad_out must be [{want[0]}, {want[1]}]")
     cnt = _host_counts("expert_count", expert_count, n_expert)
     pre = buf_pre if buf_pre is not None else buf_mid
     dev, dty = grad_out.device, grad_out.dtype
     new = lambda *s: torch.empty(*s, dtype=dty, device=dev)
-    g_out, g_mid, g_in = new(n_rows, d_model), new(n_rows, d_hidden), new(n_rows, d_model)
+    g_out = new(n_rows, d_model) if slot_order else grad_out
+    g_mid, g_in = new(n_rows, d_hidden), new(n_rows, d_model)
     grad_inp = new(n_tokens, d_model)
     grad_w1, grad_w2 = torch.empty_like(w1), torch.empty_like(w2)
     grad_b1 = torch.empty_like(b1) if b1 is not None else None
     grad_b2 = torch.empty_like(b2) if b2 is not None else None
     with torch.cuda.device(dev):
         check(_lib.load().fmoe_fused_mlp_backward(
-            ctypes.byref(prm), _ptr(grad_out), _ptr(pos), _ptr(slot_to_row), ctypes.c_void_p(cnt.data_ptr()),
+            ctypes.byref(prm), _ptr(grad_out if slot_order else None), _ptr(pos), _ptr(slot_to_row),
+            ctypes.c_void_p(cnt.data_ptr()),
             n_tokens, top_k, n_rows, _ptr(buf_in), _ptr(pre), _ptr(buf_mid), _ptr(g_out), _ptr(g_mid), _ptr(g_in),
             _ptr(grad_inp), _ptr(grad_w1), _ptr(grad_b1), _ptr(grad_w2), _ptr(grad_b2), n_chunks,
             _stream(grad_out)))

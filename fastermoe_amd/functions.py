@@ -187,6 +187,29 @@ class MOECombine(Function):
         return grad_x, grad_score.view(score_shape), None, None
 
 
+class MOEGatherCombine(Function):
+    r"""``MOEGather`` (fmoe/functions.py:285-312) and the ``bmm`` with the gate scores
+    (fmoe/layers.py:321-322) as one pass over the experts' output in expert-sorted
+    order: ``out[t] = sum_j score[t,j] * rows[slot_to_row[t*k+j]]``; dropped slots
+    (``slot_to_row < 0``) contribute zero, as the zero rows of ``_local_gather`` do."""
+
+    @staticmethod
+    def forward(ctx, rows, slot_to_row, gate_score, n_tokens, top_k):
+        rows = rows.contiguous()
+        gate_score = gate_score.contiguous()
+        ctx.save_for_backward(rows, slot_to_row, gate_score)
+        ctx.moe_args = n_tokens, top_k, gate_score.shape
+        return fmoe_native.gather_combine_forward(rows, slot_to_row, gate_score, n_tokens, top_k)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        rows, slot_to_row, gate_score = ctx.saved_tensors
+        n_tokens, top_k, score_shape = ctx.moe_args
+        grad_rows, grad_score = fmoe_native.gather_combine_backward(grad_out.contiguous(), rows, slot_to_row,
+                                                                    gate_score, n_tokens, top_k)
+        return grad_rows, None, grad_score.view(score_shape), None, None
+
+
 class AllGather(Function):
     r"""fmoe/functions.py:333-349 (model-parallel group); one worker only."""
 

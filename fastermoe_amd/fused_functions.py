@@ -41,21 +41,23 @@ def fuse_chunks():
 
 class _FusedExpertMLP(Function):
     @staticmethod
-    def forward(ctx, inp, w1, b1, w2, b2, pos, slot_to_row, expert_count, top_k, activation, n_chunks):
+    def forward(ctx, inp, w1, b1, w2, b2, pos, slot_to_row, expert_count, top_k, activation, n_chunks,
+                slot_order=True):
         out, buf_in, buf_pre, buf_mid = fmoe_native.fused_mlp_forward(
-            inp.contiguous(), pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k, activation, n_chunks)
+            inp.contiguous(), pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k, activation, n_chunks,
+            slot_order)
         ctx.save_for_backward(pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid)
-        ctx.moe_args = inp.shape[0], top_k, activation, n_chunks
+        ctx.moe_args = inp.shape[0], top_k, activation, n_chunks, slot_order
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid = ctx.saved_tensors
-        n_tokens, top_k, activation, n_chunks = ctx.moe_args
+        n_tokens, top_k, activation, n_chunks, slot_order = ctx.moe_args
         grad_inp, gw1, gb1, gw2, gb2 = fmoe_native.fused_mlp_backward(
             grad_out.contiguous(), pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid,
-            n_tokens, top_k, activation, n_chunks)
-        return grad_inp, gw1, gb1, gw2, gb2, None, None, None, None, None, None
+            n_tokens, top_k, activation, n_chunks, slot_order)
+        return grad_inp, gw1, gb1, gw2, gb2, None, None, None, None, None, None, None
 
 
 class MOEForward:
@@ -67,7 +69,10 @@ class MOEForward:
 
     @staticmethod
     def apply(inp, models, pos_s, pos_g, local_expert_count, global_expert_count, stored_models,
-              fwd_batch_size, out_batch_size, world_size, slot_to_row=None):
+              fwd_batch_size, out_batch_size, world_size, slot_to_row=None, slot_order=True):
+        r"""``slot_order=False`` (not in the reference): skip the copy back to slot order and
+        return the experts' output rows in expert-sorted order, for
+        :class:`fastermoe_amd.functions.MOEGatherCombine`."""
         if world_size != 1:
             raise NotImplementedError("MOEForward: one worker only")
         experts = models[0][0]
@@ -77,4 +82,4 @@ class MOEForward:
         act = _activation_code(experts.activation)
         return _FusedExpertMLP.apply(inp, experts.htoh4.weight, experts.htoh4.bias, experts.h4toh.weight,
                                      experts.h4toh.bias, pos_g, slot_to_row, global_expert_count.view(-1),
-                                     top_k, act, fuse_chunks())
+                                     top_k, act, fuse_chunks(), slot_order)

@@ -6,7 +6,7 @@ import os
 import torch
 import torch.nn as nn
 
-from .functions import (AllGather, MOECache, MOECombine, MOEGather, MOELinear, MOEScatter, Slice,
+from .functions import (AllGather, MOECache, MOECombine, MOEGather, MOEGatherCombine, MOELinear, MOEScatter, Slice,
                         _prepare_forward_ex, ensure_comm)
 from .gates import NaiveGate
 
@@ -50,9 +50,13 @@ def mark_module_parallel_comm(module, comm):
 
 
 def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_expert, world_size,
-                                 fused, enable_fuse=False):
+                                 fused, enable_fuse=False, combine_score=None):
     r"""Route, scatter, run the experts, gather (fmoe/layers.py:79-149).  Returns
-    ``(rows in slot order [N*top_k, d], stored_models)``."""
+    ``(rows in slot order [N*top_k, d], stored_models)``.
+
+    With ``combine_score`` (the gate scores ``[N, top_k]``; not in the reference) the
+    gather and the score-weighted sum over each token's ``top_k`` rows run as one pass
+    over the experts' output where it lies, and the first result is ``[N, d]``."""
     from .fused_functions import MOEForward
 
     (pos, local_expert_count, global_expert_count, all_expert_count, all_global_expert_count,
@@ -70,9 +74,14 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
         fwd_expert_count, policy_fn, experts, inp.shape[0], inp.shape[1], topk, num_expert,
         world_size, fused)
 
+    if combine_score is not None and slot_to_row.numel() != out_batch_size:
+        raise ValueError("combine_score needs one gate index per (token, k) pair")
     if enable_fuse:
         x = MOEForward.apply(inp, models, pos // topk, pos, local_expert_count, global_expert_count,
-                             stored_models, fwd_batch_size, out_batch_size, world_size, slot_to_row)
+                             stored_models, fwd_batch_size, out_batch_size, world_size, slot_to_row,
+                             combine_score is None)
+        if combine_score is not None:
+            x = MOEGatherCombine.apply(x, slot_to_row, combine_score, inp.shape[0], topk)
         return x, stored_models
 
     # ZeroGate hands back N*top_k indices as a 1-D tensor, so the slot count can
@@ -81,6 +90,8 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
     x = MOEScatter.apply(inp, pos // topk, local_expert_count, global_expert_count, stored_models,
                          fwd_batch_size, world_size, per_token, topk)
     x = expert_fn(x, models, fwd_expert_count, num_expert)
+    if combine_score is not None:
+        return MOEGatherCombine.apply(x, slot_to_row, combine_score, inp.shape[0], topk), stored_models
     x = MOEGather.apply(x, pos, local_expert_count, global_expert_count, stored_models,
                         out_batch_size, world_size,
                         slot_to_row if slot_to_row.numel() == out_batch_size else None)
@@ -196,9 +207,20 @@ class FMoE(nn.Module):
             inp = inp[mask == 0, :]
             gate_top_k_idx = gate_top_k_idx[mask == 0, :]
 
+        # Without a mask the gather and the combine with the gate scores are one pass
+        # (FMOE_FOLD_COMBINE=0 keeps them apart, as in the reference).
+        fold = (not masked and inp.is_cuda and inp.is_floating_point() and torch.is_tensor(gate_score)
+                and gate_score.dtype == inp.dtype and gate_top_k_idx.dim() == 2
+                and gate_score.numel() == gate_top_k_idx.numel() == inp.shape[0] * self.top_k
+                and os.environ.get("FMOE_FOLD_COMBINE", "1") != "0")
         fwd, _stored_models = _fmoe_general_global_forward(
             inp, gate_top_k_idx, self.expert_fn, self.policy_fn, self.experts, self.num_expert,
-            self.world_size, self.experts_fused, self.enable_fuse)
+            self.world_size, self.experts_fused, self.enable_fuse,
+            gate_score.reshape(inp.shape[0], self.top_k) if fold else None)
+        if fold:
+            if self.mp_size > 1:
+                fwd = AllGather.apply(fwd, self.mp_rank, self.mp_size, self.mp_group)
+            return fwd
 
         if masked:
             fwd = fwd.view(-1, self.top_k, self.d_model)

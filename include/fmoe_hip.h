@@ -145,6 +145,29 @@ int fmoe_combine_backward(const void *grad_out, const void *x, const void *score
                           int64_t top_k, int64_t row_elems, int dtype,
                           void *stream);
 
+/* The copy back to slot order folded into the combination:
+ * out[t,:] = sum_j score[t,j] * rows[slot_to_row[t*top_k+j],:], where rows
+ * [n_rows, row] are the experts' outputs in expert-sorted order and a
+ * negative slot_to_row entry (dropped slot) contributes nothing.  One pass in
+ * place of _local_gather in MOEGather.forward (fmoe/functions.py:77-84,
+ * 285-312) followed by torch.bmm (fmoe/layers.py:321-322). */
+int fmoe_gather_combine_forward(const void *rows, const int64_t *slot_to_row,
+                                const void *score, void *out, int64_t n_tokens,
+                                int64_t top_k, int64_t n_rows,
+                                int64_t row_elems, int dtype, void *stream);
+
+/* Its backward: grad_rows[slot_to_row[s],:] = score[s] * grad_out[s/top_k,:]
+ * for every kept slot s, grad_score[t,j] = <grad_out[t,:], rows[...]> (0 for a
+ * dropped slot).  Every row of grad_rows is written exactly once when
+ * slot_to_row, restricted to the kept slots, is one-to-one onto [0, n_rows)
+ * (as fmoe_route produces it); rows no slot maps to are left untouched. */
+int fmoe_gather_combine_backward(const void *grad_out, const void *rows,
+                                 const int64_t *slot_to_row, const void *score,
+                                 void *grad_rows, void *grad_score,
+                                 int64_t n_tokens, int64_t top_k,
+                                 int64_t n_rows, int64_t row_elems, int dtype,
+                                 void *stream);
+
 /* ---- per-expert linear (one grouped GEMM over ragged row segments) ------ */
 
 /* y[seg_e,:] = x[seg_e,:] . w[e]^T (+ bias[e]); seg_e are consecutive row
@@ -197,7 +220,9 @@ int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert,
  *   buf_pre    [n_rows, d_hidden]  pre-activation   (kept for backward)
  *   buf_mid    [n_rows, d_hidden]  post-activation  (kept for backward)
  *   buf_out    [n_rows, d_model]   expert output
- *   out        [n_tokens*top_k, d_model]  zero rows for dropped slots
+ *   out        [n_tokens*top_k, d_model]  zero rows for dropped slots; NULL:
+ *              the copy to slot order is skipped and the caller reads buf_out
+ *              (e.g. with fmoe_gather_combine_forward)
  * Replaces fmoe_cuda_fused_forward_impl at one worker,
  * cuda/fused_compute.cuh:250-388 (fmoe_cuda.fused_forward) together with the
  * _local_scatter/_local_gather around it, fmoe/fused_functions.py:22-32. */
@@ -208,7 +233,9 @@ int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
                            void *buf_pre, void *buf_mid, void *buf_out,
                            void *out, int n_chunks, void *stream);
 
-/* Backward of the same pipeline.  grad_out [n_tokens*top_k, d_model].
+/* Backward of the same pipeline.  grad_out [n_tokens*top_k, d_model]; NULL: the
+ * caller has already put the gradient rows in expert-sorted order into g_out
+ * (e.g. with fmoe_gather_combine_backward).
  * Scratch (caller-allocated): g_out [n_rows,d_model], g_mid [n_rows,d_hidden],
  * g_in [n_rows,d_model].  Results: grad_inp [n_tokens,d_model], grad_w1/2,
  * grad_b1/2 (bias grads may be NULL).  Weight grads of an expert split across

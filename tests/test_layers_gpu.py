@@ -105,6 +105,39 @@ def test_transformer_mlp_configs(fuse, dtype, n, d, h, e, k, act, device):
     _compare(moe, x, act, k, dtype)
 
 
+@pytest.mark.parametrize("fuse", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_folded_combine_equals_gather_then_combine(fuse, dtype, device, monkeypatch):
+    """The layer folds MOEGather and the bmm with the gate scores into one pass; with
+    FMOE_FOLD_COMBINE=0 it runs them apart as fmoe/layers.py:139-149,321-322 does.  Output, input
+    gradient, expert and gate gradients agree (dropped slots, an expert without tokens)."""
+    torch.manual_seed(5)
+    n, d, h, e, k = 257, 128, 192, 5, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe.enable_fuse = fuse
+    moe = moe.to(dtype).to(device)
+    x = torch.randn(n, d).to(dtype).to(device)
+    idx = torch.randint(0, e - 1, (n, k), device=device)
+    idx[torch.rand(n, k, device=device) < 0.2] = -1
+    gate_linear = moe.gate.gate
+
+    def gate_forward(inp):  # scores that depend on the input, so that their gradient is exercised
+        return idx, torch.softmax(gate_linear(inp)[:, :k].float(), dim=-1).to(dtype)
+
+    moe.gate.forward = gate_forward
+    results = []
+    for fold in ("0", "1"):
+        monkeypatch.setenv("FMOE_FOLD_COMBINE", fold)
+        moe.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        out.float().mean().backward()
+        results.append([out, xi.grad, gate_linear.weight.grad.clone()] + [p.grad.clone() for p in moe.experts.parameters()])
+    tol = TOL[dtype]
+    for a, b in zip(*results):
+        assert rel_err(a, b) <= tol
+
+
 @pytest.mark.parametrize("chunks", ["1", "3", "7"])
 def test_fused_equals_unfused(chunks, device, monkeypatch):
     """tests/test_fused.py:9-34 (forward, input grad, both weight grads within 1e-3),

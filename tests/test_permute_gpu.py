@@ -129,6 +129,38 @@ def test_combine_matches_bmm(dtype, n, k, d, device):
         assert (got.double().cpu() - want).abs().max() <= tol * max(1.0, want.abs().max().item())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,k,d,e,drop", [(300, 2, 1024, 8, 0.2), (64, 8, 40, 16, 0.5), (17, 3, 7, 4, 0.0),
+                                          (5, 1, 16, 3, 1.0)])
+def test_gather_combine_matches_gather_then_bmm(dtype, n, k, d, e, drop, device):
+    """The folded gather + combine and its backward against _local_gather (zero rows for
+    dropped slots, fmoe/functions.py:77-84) followed by torch.bmm (fmoe/layers.py:321-322),
+    both in float64 on the CPU."""
+    from fastermoe_amd.functions import MOEGatherCombine
+    gate, pos, s2r = _route(n, k, e, drop, n * 31 + d, device)
+    n_rows = pos.numel()
+    g = torch.Generator().manual_seed(n * k + d)
+    rows = torch.randn(n_rows, d, generator=g).to(dtype)
+    score = torch.randn(n, k, generator=g).to(dtype)
+    go = torch.randn(n, d, generator=g).to(dtype)
+    r64 = rows.detach().clone().double().requires_grad_(True)
+    s64 = score.detach().clone().double().requires_grad_(True)
+    slots = torch.zeros(n * k, d, dtype=torch.float64).index_copy(0, pos.cpu(), r64)
+    ref = torch.bmm(s64.view(n, 1, k), slots.view(n, k, d)).reshape(n, d)
+    ref.backward(go.double())
+    rd = rows.detach().to(device).requires_grad_(True)
+    sd = score.detach().to(device).requires_grad_(True)
+    out = MOEGatherCombine.apply(rd, s2r, sd, n, k)
+    out.backward(go.to(device))
+    tol = {torch.float32: 1e-5, torch.float64: 1e-12}.get(dtype, 2e-2)
+    for got, want in ((out, ref), (rd.grad, r64.grad), (sd.grad, s64.grad)):
+        assert got.shape == want.shape
+        if want.numel():
+            assert (got.double().cpu() - want).abs().max() <= tol * max(1.0, want.abs().max().item())
+    # dropped slots get a zero score gradient
+    assert torch.count_nonzero(sd.grad.view(-1)[s2r < 0]) == 0
+
+
 def test_full_size_round_trip(device):
     """config-4 sized rows: scatter then gather restores every kept slot, dropped slots are zero;
     linearity of the reduction."""
