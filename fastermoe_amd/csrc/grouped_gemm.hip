@@ -58,9 +58,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_plain_kernel(const Gemm
         if (bias) acc += (Acc)bias[col];
         if (prm.epilogue == kEpiBiasAct) {
             if (prm.aux) ((T *)prm.aux)[c_off] = (T)acc;
-            acc = (Acc)apply_act((float)acc, prm.activation);
+            acc = (Acc)apply_act<false>((float)acc, prm.activation);
         } else if (prm.epilogue == kEpiDAct) {
-            acc *= (Acc)act_grad((float)((const T *)prm.aux)[c_off], prm.activation);
+            acc *= (Acc)act_grad<false>((float)((const T *)prm.aux)[c_off], prm.activation);
         }
         if (accumulate) acc += (Acc)*dst;
         *dst = (T)acc;

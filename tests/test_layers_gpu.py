@@ -351,3 +351,39 @@ def test_fused_many_experts_few_rows(chunks, device, monkeypatch):
     ref = _oracle(moe, x, idx, score, "relu", k)
     assert rel_err(results[1][0], ref["out"]) <= 1e-5
     assert rel_err(results[1][2], ref["grad_w1"]) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_fused_gelu_epilogue_accuracy(dtype, device):
+    """The activation computed in the GEMM epilogue against torch's exact (erf) GELU of the
+    saved pre-activation, over pre-activations from -9 to 9: within one rounding step of the
+    element type (relative), plus 1e-4 absolute for the far negative tail where GELU -> 0;
+    and the derivative used by the backward against autograd's."""
+    from fastermoe_amd import _lib, fmoe_native
+    n, d, h = 512, 64, 256
+    x = torch.randn(n, d, device=device).to(dtype)
+    w1 = (torch.randn(1, h, d, device=device) * 0.4).to(dtype)      # pre-activations ~ N(0, 3.2^2)
+    b1 = torch.linspace(-6, 6, h, device=device).view(1, h).to(dtype)
+    w2 = torch.eye(h, device=device).view(1, h, h)[:, :d, :].contiguous().to(dtype)  # picks the first d hidden units
+    pos = torch.arange(n, device=device)
+    cnt = torch.tensor([n])
+    out, buf_in, buf_pre, buf_mid = fmoe_native.fused_mlp_forward(x, pos, pos.clone(), cnt, w1, b1, w2, None, 1,
+                                                                  _lib.ACT_GELU, 1)
+    pre = buf_pre.float()
+    assert pre.min() < -6 and pre.max() > 6
+    want = torch.nn.functional.gelu(pre)
+    step = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -20}[dtype]
+    # buf_pre is the rounded pre-activation, the kernel activates the unrounded one: allow that rounding too
+    slack = step * pre.abs() * 1.13  # |GELU'| <= 1.13
+    assert ((buf_mid.float() - want).abs() <= 2 * step * want.abs() + slack + 1e-4).all()
+    # derivative: grad of sum(mid) w.r.t. pre through the library's backward = GELU'(pre)
+    pre_leaf = pre.clone().requires_grad_(True)
+    torch.nn.functional.gelu(pre_leaf).sum().backward()
+    grad_inp, gw1, gb1, gw2, gb2 = fmoe_native.fused_mlp_backward(
+        torch.ones(n, d, device=device, dtype=dtype), pos, pos.clone(), cnt, w1, b1, w2, None, buf_in, buf_pre,
+        buf_mid, n, 1, _lib.ACT_GELU, 1)
+    # gb1[j] = sum_rows g_mid[:, j] with g_mid = (ones . W2)[:, j] * GELU'(pre[:, j]); W2 picks the first d units
+    want_gb1 = (pre_leaf.grad[:, :d]).sum(0)
+    got_gb1 = gb1.float().view(-1)[:d]
+    assert ((got_gb1 - want_gb1).abs() <= 4 * step * want_gb1.abs() + 0.05 * step * n).all()
+    assert torch.count_nonzero(gb1.float().view(-1)[d:]) == 0
