@@ -11,7 +11,10 @@
 // exit, so the call behaves like one asynchronous operation on that stream.
 // Backward mirrors this: gather grad rows, dgrad/wgrad of both linears with the
 // activation derivative folded into the first dgrad's epilogue, and a final
-// per-token reduction of the k expert-row gradients.
+// per-token reduction of the k expert-row gradients.  A caller that combines the
+// experts' outputs straight from the sorted buffer passes out = NULL (no
+// permute-out stage), and grad_out = NULL in the backward when it has already
+// written the gradient rows in sorted order (no permute-in stage).
 //
 // All streams use the default priority.  Events are created once per device and
 // reused; a call therefore must not overlap another call of this library's fused
