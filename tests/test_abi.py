@@ -30,6 +30,34 @@ def test_library_exports_every_declared_symbol():
     assert lib.fmoe_abi_version() == 1
 
 
+def test_ctypes_signatures_match_the_header():
+    """Every prototype in include/fmoe_hip.h against the ctypes table: same number of parameters,
+    pointers where the header has pointers, 64-bit integers where it has int64_t, int where it has
+    int -- a mismatch would silently corrupt the arguments of a call."""
+    import ctypes
+    text = open(os.path.join(ROOT, "include", "fmoe_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    protos = re.findall(r"\b([a-z0-9_ ]+?[ \*])(fmoe_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text)
+    assert len(protos) == len(_lib.SIGNATURES)
+    for ret, name, params in protos:
+        restype, argtypes = _lib.SIGNATURES[name]
+        params = [q.strip() for q in params.split(",") if q.strip() and q.strip() != "void"]
+        assert len(params) == len(argtypes), f"{name}: header has {len(params)} parameters, ctypes table {len(argtypes)}"
+        for q, a in zip(params, argtypes):
+            if "*" in q:
+                assert a is ctypes.c_void_p or issubclass(a, ctypes._Pointer), f"{name}: `{q}` is a pointer"
+            elif q.startswith("int64_t"):
+                assert a is ctypes.c_int64, f"{name}: `{q}` is int64_t"
+            else:
+                assert q.startswith("int ") and a is ctypes.c_int, f"{name}: `{q}`"
+        if "*" in ret:
+            assert restype in (ctypes.c_char_p, ctypes.c_void_p)
+        elif "int64_t" in ret:
+            assert restype is ctypes.c_int64
+        else:
+            assert restype is ctypes.c_int
+
+
 def test_workspace_queries_run_without_a_gpu():
     lib = _lib.load()
     assert lib.fmoe_routing_workspace_bytes(65536, 256) >= (32 * 256 + 512) * 4
