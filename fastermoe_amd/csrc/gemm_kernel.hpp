@@ -398,6 +398,30 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                    (uint32_t)(Q_BASE + buf * Q_BYTES));
     };
 
+    // Data-grad with the activation derivative, 16-bit types: the tile of saved
+    // pre-activations that the epilogue needs (BM rows x 512 bytes) is requested in the load
+    // slots of the last two slabs, whose own loads would only fetch zeros past the end of
+    // the contraction -- 64 rows (one P buffer's worth) per slot, parts 0 and 1 in the P slots,
+    // parts 2 and 3 (256-row tiles) in the Q slots -- so it lands while the last MFMAs run
+    // instead of after them, when every workgroup of the round asks memory at once.
+    // Slot q of a part is row q/32, position q%32, and holds chunk (q%32) ^ (row%16).
+    constexpr bool kAuxPrefetch = EPI == kEpiDAct && sizeof(T) == 2 && kDmaAsm && BN == 256;
+    constexpr int kAuxParts = BM / 64;
+    const T *aux_tile = (const T *)prm.aux + aux_off;
+    auto issue_aux = [&](int part, uint32_t lds_off) {
+        if constexpr (kAuxPrefetch) {
+#pragma unroll
+            for (int it = 0; it < NP; ++it) {
+                const int rip = it * 8 + (t >> 5);              // row inside the part
+                const int row = part * 64 + rip;
+                const int c = (t & 31) ^ (rip & 15);
+                const bool ok = row < q_valid && c * CE < p_valid;
+                const uint32_t voff = ok ? (uint32_t)(((int64_t)row * prm.ldc + c * CE) * sizeof(T)) : kOutOfRange;
+                dma_asm(aux_tile, (int64_t)kOutOfRange, lds_off + wave_u * 1024 + it * kPassBytes, voff);
+            }
+        }
+    };
+
     // Bias gradient (weight-gradient product only): the workgroups of the first column
     // tile also add up the rows of the Q slabs they stage, i.e. the column sums of the
     // output gradient over the expert's rows.  Every thread keeps the sums of the CE
@@ -510,6 +534,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     auto phase_reads = [&](int ph) { return PF * kPReadsPerFrag + (phase_reads_q(ph) ? TJ * kQReadsPerFrag : 0); };
 
     const int n_slabs = (K + BKE - 1) / BKE;
+    const bool aux_pref = kAuxPrefetch && n_slabs >= 2;  // both tail slabs exist
     u32x4 pf[2][PF], qf[2][TJ];
     // the fragments of phase ph, in the order its MFMAs (x outer, y inner) first need them
     auto read_phase = [&](int ph, const unsigned char *sp, const unsigned char *sq) {
@@ -565,7 +590,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             const unsigned char *sq = smem + Q_BASE + (s & 1) * Q_BYTES;
 #pragma unroll
             for (int ph = 0; ph + 1 < kPhases; ++ph) {
-                if (kLoads && ph == 0) issue_p((s + 2) * BKE, pf_buf);
+                if (kLoads && ph == 0) {
+                    const int past_end = s + 2 - n_slabs;  // >= 0: slab s+2 does not exist
+                    if (kAuxPrefetch && aux_pref && past_end >= 0) issue_aux(past_end, (uint32_t)(pf_buf * P_BYTES));
+                    else issue_p((s + 2) * BKE, pf_buf);
+                }
                 read_phase(ph + 1, sp, sq);
                 mma_phase(ph, 0, PF);
 #pragma unroll
@@ -579,7 +608,13 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             wait_loads(std::integral_constant<int, kLoads ? NP : kNoWait>{});  // everything but the P loads of slab s+2
             slab_barrier();
             if constexpr (kBias) add_q_chunks((s + 1) & 1);
-            if constexpr (kLoads) issue_q((s + 2) * BKE, s & 1);
+            if constexpr (kLoads) {
+                const int past_end = s + 2 - n_slabs;
+                if (kAuxPrefetch && kAuxParts == 4 && aux_pref && past_end >= 0)
+                    issue_aux(2 + past_end, (uint32_t)(Q_BASE + (s & 1) * Q_BYTES));
+                else
+                    issue_q((s + 2) * BKE, s & 1);
+            }
             read_phase(0, smem + pn * P_BYTES, smem + Q_BASE + ((s + 1) & 1) * Q_BYTES);
             mma_phase(kPhases - 1, 0, PF);
             constexpr int kQLoadsPerMfma = (NQ + kMfma - 1) / kMfma;
@@ -694,11 +729,37 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         for (int i = 0; i < 4; ++i) v[i] = (float)in[i];
     };
 
-    // The activation and the accumulate flag are fixed per launch; the epilogue is instantiated
-    // per value so that its element loop is straight-line code.
-    auto run_epilogue = [&](auto act_tag, auto accum_tag) {
+    // The pre-activation tile that was requested during the last two slabs lies in the slab
+    // buffers; every lane takes the 4 values per block it needs into registers (the fragment
+    // registers are free now) before the staging area, which overlaps those buffers, is used.
+    u32x2 auxv[kAuxPrefetch ? TI : 1][kAuxPrefetch ? TJ : 1];
+    if constexpr (kAuxPrefetch) {
+        if (aux_pref) {
+            // part 0 / 1 went to the P buffers that slabs n-2 / n-1 would have prefetched into,
+            // part 2 / 3 to the Q buffers of slabs n-2 / n-1
+            const int row_t = wave_m0 + lb;                // tile row of this lane in block row 0
+            const int part = row_t >> 6;                   // the same for all block rows of the wave
+            const uint32_t part_off = part < 2 ? (uint32_t)(((n_slabs + part) % kPBufs) * P_BYTES)
+                                               : (uint32_t)(Q_BASE + ((n_slabs + part) & 1) * Q_BYTES);
+#pragma unroll
+            for (int x = 0; x < TI; ++x)
+#pragma unroll
+                for (int y = 0; y < TJ; ++y) {
+                    const int rip = (row_t & 63) + y * MB;
+                    const int c = ((wave_n0 + x * MB) >> 3) + (hq >> 1);
+                    auxv[x][y] = *(const u32x2 *)(smem + part_off + rip * 512 + ((c ^ (rip & 15)) << 4) + (hq & 1) * 8);
+                }
+            __syncthreads();
+        }
+    }
+
+    // The activation, the accumulate flag and where the tile that is read comes from are fixed
+    // per launch (per tile); the epilogue is instantiated per value so that its element loop is
+    // straight-line code.
+    auto run_epilogue = [&](auto act_tag, auto accum_tag, auto auxreg_tag) {
     constexpr int ACT = decltype(act_tag)::value;
     constexpr bool kAccum = decltype(accum_tag)::value;
+    constexpr bool kAuxRegs = decltype(auxreg_tag)::value;  // the pre-activations are in auxv
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
         const int col_base = wave_n0 + pass * CPP;
@@ -708,7 +769,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         for (int kind = kKinds - 1; kind >= 0; --kind) {
             if (EPI == kEpiBiasAct && kind == 1 && !aux) continue;
             constexpr bool reads_tile = (EPI == kEpiDAct) || kAccum;
-            if (reads_tile) {
+            if (reads_tile && !kAuxRegs) {
                 stage_in(EPI == kEpiDAct ? (const T *)aux : (const T *)Cb, col_base);
                 lds_sync();
             }
@@ -738,7 +799,14 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                         }
                         if (reads_tile) {
                             float in[4];
-                            get4(row, cip, in);
+                            if constexpr (kAuxRegs) {
+                                alignas(8) T a4[4];
+                                *(u32x2 *)a4 = auxv[kAuxPrefetch ? x : 0][kAuxPrefetch ? y : 0];
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) in[i] = (float)a4[i];
+                            } else {
+                                get4(row, cip, in);
+                            }
 #pragma unroll
                             for (int i = 0; i < 4; ++i)
                                 v[i] = (EPI == kEpiDAct) ? v[i] * act_grad<sizeof(T) == 2>(in[i], ACT) : v[i] + in[i];
@@ -754,13 +822,19 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     }
     };
     typedef std::integral_constant<int, FMOE_ACT_NONE> ActNone;
+    auto by_activation = [&](auto auxreg_tag) {
+        if (prm.activation == FMOE_ACT_GELU) run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{}, auxreg_tag);
+        else if (prm.activation == FMOE_ACT_RELU) run_epilogue(std::integral_constant<int, FMOE_ACT_RELU>{}, std::false_type{}, auxreg_tag);
+        else run_epilogue(ActNone{}, std::false_type{}, auxreg_tag);
+    };
     if constexpr (EPI == kEpiStore) {
-        if (accumulate) run_epilogue(ActNone{}, std::true_type{});
-        else run_epilogue(ActNone{}, std::false_type{});
+        if (accumulate) run_epilogue(ActNone{}, std::true_type{}, std::false_type{});
+        else run_epilogue(ActNone{}, std::false_type{}, std::false_type{});
+    } else if constexpr (kAuxPrefetch) {
+        if (aux_pref) by_activation(std::true_type{});
+        else by_activation(std::false_type{});
     } else {
-        if (prm.activation == FMOE_ACT_GELU) run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{});
-        else if (prm.activation == FMOE_ACT_RELU) run_epilogue(std::integral_constant<int, FMOE_ACT_RELU>{}, std::false_type{});
-        else run_epilogue(ActNone{}, std::false_type{});
+        by_activation(std::false_type{});
     }
 #endif  // __HIP_DEVICE_COMPILE__
 }

@@ -138,6 +138,35 @@ def test_folded_combine_equals_gather_then_combine(fuse, dtype, device, monkeypa
         assert rel_err(a, b) <= tol
 
 
+@pytest.mark.parametrize("dtype,n,d,h,e,k", [
+    # 512+ tiles in the second data-grad: 256-row tiles, ragged row and column tails (bfloat16 only: the
+    # mean() loss of a batch this large puts float16 gradients into the subnormal range)
+    (torch.bfloat16, 4100, 256, 4104, 2, 2),
+    (torch.bfloat16, 300, 128, 520, 3, 2),     # contraction of exactly two slabs, 128-row tiles
+    (torch.float16, 300, 128, 520, 3, 2),
+    (torch.bfloat16, 300, 64, 264, 3, 2),      # one slab: no tail slabs to carry the pre-activation tile
+    (torch.float16, 300, 64, 264, 3, 2),
+    (torch.bfloat16, 700, 200, 776, 2, 1),     # three slabs and a ragged contraction tail
+    (torch.float16, 700, 200, 776, 2, 1),
+])
+def test_fused_backward_tail_slabs(dtype, n, d, h, e, k, device, monkeypatch):
+    """The second data-grad of the fused 16-bit path loads its pre-activation tile in the
+    load slots of the last two contraction slabs: shapes with one, two, three and many
+    slabs, both tile heights, ragged tails, against the float64 oracle."""
+    monkeypatch.setenv("FMOE_FUSE_GRAN", "1")
+    torch.manual_seed(n + d)
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe.enable_fuse = True
+    with torch.no_grad():
+        moe.experts.htoh4.weight.normal_(0, d ** -0.5)
+        moe.experts.h4toh.weight.normal_(0, h ** -0.5)
+        moe.experts.htoh4.bias.normal_(0, 0.5)
+        moe.experts.h4toh.bias.normal_(0, 0.1)
+    moe = moe.to(dtype).to(device)
+    x = torch.randn(n, d).to(dtype).to(device)
+    _compare(moe, x, "gelu", k, dtype)
+
+
 @pytest.mark.parametrize("chunks", ["1", "3", "7"])
 def test_fused_equals_unfused(chunks, device, monkeypatch):
     """tests/test_fused.py:9-34 (forward, input grad, both weight grads within 1e-3),
