@@ -369,7 +369,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // the chunk is dropped when it lies past K.  MC: the resource starts at contraction row
     // k0 and is exactly as long as the rows that remain, so rows past K read as zero.
     auto issue_part = [&](auto shape_tag, const T *tile, int64_t ld, int kc_chunk, const uint32_t *voff, auto n_tag, int k0,
-                          uint32_t lds_off) {
+                          uint32_t lds_off, int it_lo = 0, int it_hi = 1 << 20) {
         constexpr int SHAPE = decltype(shape_tag)::value;
         constexpr int N = decltype(n_tag)::value;
         const int k_left = K - k0;  // <= 0 past the end: everything reads as zero
@@ -381,6 +381,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         const uint32_t past = (SHAPE == kKC) ? ((uint32_t)(k_left - 1 - kc_chunk * CE) & kOutOfRange) : 0u;
 #pragma unroll
         for (int it = 0; it < N; ++it) {
+            if (it < it_lo || it >= it_hi) continue;
             if constexpr (kDmaAsm)
                 dma_asm(origin, bytes, lds_off + wave_u * 1024 + it * kPassBytes, voff[it] | past);
             else
@@ -389,9 +390,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                     voff[it] | past, 0, 0, 0);
         }
     };
-    auto issue_p = [&](int k0, int buf) {
+    auto issue_p = [&](int k0, int buf, int it_lo = 0, int it_hi = 1 << 20) {
         issue_part(std::integral_constant<int, PSHAPE>{}, Pb, prm.ldp, p_kc_chunk, p_voff, std::integral_constant<int, NP>{}, k0,
-                   (uint32_t)(buf * P_BYTES));
+                   (uint32_t)(buf * P_BYTES), it_lo, it_hi);
     };
     auto issue_q = [&](int k0, int buf) {
         issue_part(std::integral_constant<int, QSHAPE>{}, Qb, prm.ldq, q_kc_chunk, q_voff, std::integral_constant<int, NQ>{}, k0,
@@ -507,8 +508,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // of the slab's two contraction steps, so the Q fragments are read every other phase.
     // P buffer pc holds slab s, pn slab s+1, pf_buf receives slab s+2; Q buffer s%2 holds
     // slab s.  Per slab:
-    //   phase 0     : MFMAs of phase 0, LDS reads of phase 1, and the P loads of slab s+2
-    //   phases 1..2 : MFMAs of the phase, LDS reads of the next one between them
+    //   phases 0..1 : MFMAs of the phase, LDS reads of the next one, and half of the P loads
+    //                 of slab s+2 each
+    //   phase 2     : MFMAs of the phase, LDS reads of phase 3 between them
     //   wait        : until this wave's loads of slab s+1 have landed (the P loads of slab
     //                 s+2 stay in flight) and its reads of phase 3 have returned
     //   barrier     : slab s+1 is complete and nobody reads slab s any more
@@ -525,7 +527,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int kQReadsPerFrag = (QSHAPE == kMC) ? (sizeof(T) == 2 ? 2 : 4) : 1;
     constexpr int kMfma = PF * TJ * (sizeof(T) == 4 ? 4 : 1);   // MFMA instructions per phase
     constexpr int kReadsPerMfma = 1;  // a phase's reads go out early, one per MFMA; the remaining MFMAs follow
-    constexpr int kLoadsPerMfma = (NP + kMfma - 1) / kMfma;
+    static_assert(NP % 2 == 0 && NP / 2 <= kMfma, "the P loads of a slab go out in two halves, one load per MFMA");
     // contraction step, first block column, Q fragment buffer of a phase; does it start a step
     auto phase_ks = [](int ph) { return MB == 32 ? ph : ph >> 1; };
     auto phase_x0 = [](int ph) { return MB == 32 ? 0 : (ph & 1) * PF; };
@@ -593,7 +595,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                 if (kLoads && ph == 0) {
                     const int past_end = s + 2 - n_slabs;  // >= 0: slab s+2 does not exist
                     if (kAuxPrefetch && aux_pref && past_end >= 0) issue_aux(past_end, (uint32_t)(pf_buf * P_BYTES));
-                    else issue_p((s + 2) * BKE, pf_buf);
+                    else issue_p((s + 2) * BKE, pf_buf, 0, NP / 2);
+                }
+                if (kLoads && ph == 1) {  // the second half of the P loads (the pre-activation part went out whole)
+                    const int past_end = s + 2 - n_slabs;
+                    if (!(kAuxPrefetch && aux_pref && past_end >= 0)) issue_p((s + 2) * BKE, pf_buf, NP / 2, NP);
                 }
                 read_phase(ph + 1, sp, sq);
                 mma_phase(ph, 0, PF);
@@ -601,7 +607,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                 for (int i = 0; i < kMfma; ++i) {
                     if (i * kReadsPerMfma < phase_reads(ph + 1)) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);  // LDS reads
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       // one MFMA
-                    if (kLoads && ph == 0 && i * kLoadsPerMfma < NP) __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPerMfma, 0);  // loads
+                    if (kLoads && ph <= 1 && i < NP / 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
