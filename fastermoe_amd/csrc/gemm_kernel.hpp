@@ -508,9 +508,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // of the slab's two contraction steps, so the Q fragments are read every other phase.
     // P buffer pc holds slab s, pn slab s+1, pf_buf receives slab s+2; Q buffer s%2 holds
     // slab s.  Per slab:
-    //   phases 0..1 : MFMAs of the phase, LDS reads of the next one, and half of the P loads
+    //   phase 0     : MFMAs of the phase, LDS reads of phase 1 between them
+    //   phases 1..2 : MFMAs of the phase, LDS reads of the next one, and half of the P loads
     //                 of slab s+2 each
-    //   phase 2     : MFMAs of the phase, LDS reads of phase 3 between them
     //   wait        : until this wave's loads of slab s+1 have landed (the P loads of slab
     //                 s+2 stay in flight) and its reads of phase 3 have returned
     //   barrier     : slab s+1 is complete and nobody reads slab s any more
@@ -528,6 +528,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int kMfma = PF * TJ * (sizeof(T) == 4 ? 4 : 1);   // MFMA instructions per phase
     constexpr int kReadsPerMfma = 1;  // a phase's reads go out early, one per MFMA; the remaining MFMAs follow
     static_assert(NP % 2 == 0 && NP / 2 <= kMfma, "the P loads of a slab go out in two halves, one load per MFMA");
+    // phases that carry the two halves: phase 3 carries the Q loads, phase 0 is left to let
+    // the load queue drain (0 and 1 measured 0.5 % slower per step, all in phase 0 1 %)
+    constexpr int kPLoadPhaseA = 1, kPLoadPhaseB = 2;
     // contraction step, first block column, Q fragment buffer of a phase; does it start a step
     auto phase_ks = [](int ph) { return MB == 32 ? ph : ph >> 1; };
     auto phase_x0 = [](int ph) { return MB == 32 ? 0 : (ph & 1) * PF; };
@@ -592,12 +595,12 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             const unsigned char *sq = smem + Q_BASE + (s & 1) * Q_BYTES;
 #pragma unroll
             for (int ph = 0; ph + 1 < kPhases; ++ph) {
-                if (kLoads && ph == 0) {
+                if (kLoads && ph == kPLoadPhaseA) {
                     const int past_end = s + 2 - n_slabs;  // >= 0: slab s+2 does not exist
                     if (kAuxPrefetch && aux_pref && past_end >= 0) issue_aux(past_end, (uint32_t)(pf_buf * P_BYTES));
                     else issue_p((s + 2) * BKE, pf_buf, 0, NP / 2);
                 }
-                if (kLoads && ph == 1) {  // the second half of the P loads (the pre-activation part went out whole)
+                if (kLoads && ph == kPLoadPhaseB) {  // the second half of the P loads (the pre-activation part went out whole)
                     const int past_end = s + 2 - n_slabs;
                     if (!(kAuxPrefetch && aux_pref && past_end >= 0)) issue_p((s + 2) * BKE, pf_buf, NP / 2, NP);
                 }
@@ -607,7 +610,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
                 for (int i = 0; i < kMfma; ++i) {
                     if (i * kReadsPerMfma < phase_reads(ph + 1)) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerMfma, 0);  // LDS reads
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                       // one MFMA
-                    if (kLoads && ph <= 1 && i < NP / 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
+                    if (kLoads && (ph == kPLoadPhaseA || ph == kPLoadPhaseB) && i < NP / 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
