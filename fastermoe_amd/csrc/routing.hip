@@ -18,6 +18,8 @@
 // three short launches with coalesced 8-byte loads.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace fmoe {
 namespace {
 
@@ -339,21 +341,12 @@ extern "C" int fmoe_assign_pos(int32_t *cum_count, const int64_t *gate, int64_t 
     return FMOE_OK;
 }
 
-extern "C" int fmoe_route(const int64_t *gate, int64_t n_slots, int64_t n_expert, int64_t *expert_count,
-                          int64_t *pos, int64_t *slot_to_row, void *workspace, int64_t workspace_bytes,
-                          void *stream) {
-    if (int rc = check_sizes(n_slots, n_expert)) return rc;
-    FMOE_REQUIRE(expert_count, "fmoe_route: NULL expert_count");
-    hipStream_t st = (hipStream_t)stream;
-    if (n_slots == 0) {
-        // a fill kernel, not hipMemsetAsync, so that the call can be captured into a HIP graph
-        zero_counts_kernel<<<(int)ceil_div(n_expert, kBlock), kBlock, 0, st>>>(expert_count, n_expert);
-        FMOE_LAUNCH_CHECK();
-        return FMOE_OK;
-    }
-    FMOE_REQUIRE(gate && pos, "fmoe_route: NULL pointer");
-    RouteScratch s;
-    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+namespace fmoe {
+namespace {
+
+// histogram -> scan over workgroups and experts -> placement, on scratch carved by the caller
+int route_launch(const int64_t *gate, int64_t n_slots, int64_t n_expert, int64_t *expert_count, int64_t *pos,
+                 int64_t *slot_to_row, const RouteScratch &s, hipStream_t st) {
     const int E = (int)n_expert;
     block_hist_kernel<<<s.n_blocks, kBlock, E * sizeof(int32_t), st>>>(gate, s.block_hist, n_slots, E);
     FMOE_LAUNCH_CHECK();
@@ -363,6 +356,76 @@ extern "C" int fmoe_route(const int64_t *gate, int64_t n_slots, int64_t n_expert
         gate, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert));
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
+}
+
+int route_empty(int64_t n_expert, int64_t *expert_count, hipStream_t st) {
+    // a fill kernel, not hipMemsetAsync, so that the call can be captured into a HIP graph
+    zero_counts_kernel<<<(int)ceil_div(n_expert, kBlock), kBlock, 0, st>>>(expert_count, n_expert);
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+// Scratch of fmoe_route_static: a fixed device array instead of a caller's workspace, so
+// that the entry point never allocates.  Every GPU holds its own copy at its own address;
+// `scratch` is only the host-side handle of the symbol, the device address is looked
+// up once per device and kept in g_static_scratch_ptr.
+constexpr int64_t kStaticScratchBytes = FMOE_ROUTE_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 16;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+std::mutex g_static_scratch_mutex;
+void *g_static_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch_address(void **out) {
+    int dev = 0;
+    FMOE_HIP_CHECK(hipGetDevice(&dev));
+    FMOE_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (g_static_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        FMOE_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        FMOE_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned NULL for the routing scratch");
+        g_static_scratch_ptr[dev] = ptr;
+    }
+    *out = g_static_scratch_ptr[dev];
+    return FMOE_OK;
+}
+
+}  // namespace
+}  // namespace fmoe
+
+extern "C" int fmoe_route(const int64_t *gate, int64_t n_slots, int64_t n_expert, int64_t *expert_count,
+                          int64_t *pos, int64_t *slot_to_row, void *workspace, int64_t workspace_bytes,
+                          void *stream) {
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    FMOE_REQUIRE(expert_count, "fmoe_route: NULL expert_count");
+    hipStream_t st = (hipStream_t)stream;
+    if (n_slots == 0) return route_empty(n_expert, expert_count, st);
+    FMOE_REQUIRE(gate && pos, "fmoe_route: NULL pointer");
+    RouteScratch s;
+    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+    return route_launch(gate, n_slots, n_expert, expert_count, pos, slot_to_row, s, st);
+}
+
+extern "C" int fmoe_route_static(const int64_t *gate, int64_t n_slots, int64_t n_expert, int64_t *expert_count,
+                                 int64_t *pos, int64_t *slot_to_row, void *stream) {
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    FMOE_REQUIRE(expert_count, "fmoe_route_static: NULL expert_count");
+    hipStream_t st = (hipStream_t)stream;
+    if (n_slots == 0) return route_empty(n_expert, expert_count, st);
+    FMOE_REQUIRE(gate && pos, "fmoe_route_static: NULL pointer");
+    const int64_t need = scratch_bytes(n_slots, n_expert);
+    if (need > kStaticScratchBytes)
+        return fail(FMOE_ELIMIT,
+                    "fmoe_route_static: %lld slots x %lld experts need %lld bytes of scratch, the built-in "
+                    "array holds %lld; use fmoe_route with a workspace",
+                    (long long)n_slots, (long long)n_expert, (long long)need, (long long)kStaticScratchBytes);
+    void *scratch_dev = nullptr;
+    if (int rc = static_scratch_address(&scratch_dev)) return rc;
+    RouteScratch s;
+    if (int rc = carve(scratch_dev, kStaticScratchBytes, n_slots, n_expert, &s)) return rc;
+    // Every cell of the scratch that the scan and the placement read is written by the
+    // histogram / scan launched just before them, so nothing has to be cleared between calls.
+    return route_launch(gate, n_slots, n_expert, expert_count, pos, slot_to_row, s, st);
 }
 
 extern "C" int fmoe_limit_by_capacity(const int64_t *ec, int32_t *cap, int64_t *eca, int64_t n_expert,

@@ -78,6 +78,22 @@ int fmoe_route(const int64_t *gate, int64_t n_slots, int64_t n_expert,
                int64_t *expert_count, int64_t *pos, int64_t *slot_to_row,
                void *workspace, int64_t workspace_bytes, void *stream);
 
+/* fmoe_route for callers that must not allocate (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc): same inputs, outputs and
+ * results as fmoe_route, but the scratch is a fixed array of
+ * FMOE_ROUTE_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held
+ * until the process ends) instead of a caller's workspace, and the call makes
+ * no hipMalloc / hipFree.  Sizes with
+ * fmoe_routing_workspace_bytes(n_slots, n_expert) above that limit return
+ * FMOE_ELIMIT.  All calls on one GPU share the array: calls that overlap in
+ * time on one GPU (different streams or host threads) race.  The first call on
+ * a device looks up the array's device address (hipGetSymbolAddress); make it
+ * outside any stream capture.  No counterpart in the reference. */
+#define FMOE_ROUTE_STATIC_SCRATCH_BYTES (1 << 20)
+int fmoe_route_static(const int64_t *gate, int64_t n_slots, int64_t n_expert,
+                      int64_t *expert_count, int64_t *pos,
+                      int64_t *slot_to_row, void *stream);
+
 /* ---- capacity balancing ------------------------------------------------- */
 
 /* eca[w,e] = share of cap[e] granted to worker w, workers served in ascending
