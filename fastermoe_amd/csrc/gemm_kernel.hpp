@@ -6,6 +6,7 @@
 #include "profile.hpp"
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 namespace fmoe {
@@ -153,6 +154,14 @@ struct GemmParams {
     int32_t activation;
     int32_t accumulate_first;  // ragged-K: expert 0 of the table adds to C
     int32_t epilogue;          // Epilogue, read by the any-shape kernel only
+    // Ragged rows only.  The tiles beyond the last whole round of the chip (tiles main_tiles ..
+    // total_tiles - 1 of the logical order) can be split along the contraction: k_split
+    // workgroups compute split_slabs slabs each and leave their fp32 accumulators in split_ws;
+    // split_reduce_kernel then adds the parts of every tile in ascending order into part 0, and a
+    // second launch of this kernel (fixup != 0, one wave per workgroup) loads the sums and runs
+    // the epilogue.  k_split == 1: main_tiles == total_tiles.
+    float *split_ws;
+    int32_t main_tiles, k_split, split_slabs, fixup;
     int32_t block_m;           // host only: tile height the segment table was built for (256 or 128)
     int32_t profile_class;     // host only: ProfileClass of this launch
     double profile_work;       // host only: flop of this launch
@@ -193,12 +202,27 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // tile costs as much as its expert has rows, so every XCD takes a contiguous eighth of
     // EACH expert's tiles instead -- skewed routing then loads the XCDs evenly.
     int ei, mt, nt;
+    int split_part = -1;   // >= 0: this workgroup computes that part of the contraction of a tail tile
+    int tail_index = 0;    // index of a tail tile among the tail tiles
+    const bool fixup = RAGGED == kRaggedRows && prm.fixup != 0;
     {
         int tm_total, rem;
         if (RAGGED == kRaggedRows) {
-            const int per_xcd = (gridDim.x + 7) >> 3;
-            const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-            if (L >= prm.total_tiles) return;
+            int L;
+            const int main_grid = (prm.main_tiles + 7) & ~7;
+            if (fixup) {
+                tail_index = blockIdx.x >> 3;  // eight one-wave workgroups per tail tile
+                L = prm.main_tiles + tail_index;
+            } else if ((int)blockIdx.x < main_grid) {
+                const int per_xcd = main_grid >> 3;
+                L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+                if (L >= prm.main_tiles) return;
+            } else {
+                const int u = blockIdx.x - main_grid, n_tail = prm.total_tiles - prm.main_tiles;
+                split_part = u / n_tail;
+                tail_index = u - split_part * n_tail;
+                L = prm.main_tiles + tail_index;
+            }
             tm_total = prm.tab.tile[prm.tab.n];
             rem = L;
             ei = 0;
@@ -244,6 +268,12 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         const T *Pe = (const T *)prm.P + (int64_t)expert * prm.p_expert_stride;
         Pb = (PSHAPE == kKC) ? Pe + (int64_t)n0 * prm.ldp : Pe + n0;
         aux_off = (int64_t)row0 * prm.ldc + n0;
+        if (split_part >= 0) {  // this part's slabs only
+            const int k_begin = split_part * prm.split_slabs * BKE;
+            K = max(0, min(K - k_begin, prm.split_slabs * BKE));
+            Qb += (QSHAPE == kKC) ? (int64_t)k_begin : (int64_t)k_begin * prm.ldq;
+            Pb += (PSHAPE == kKC) ? (int64_t)k_begin : (int64_t)k_begin * prm.ldp;
+        }
     } else {
         const int m0 = mt * BM;
         q_valid = min(BM, prm.n_rows - m0);
@@ -256,7 +286,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     Cb = (T *)prm.C + aux_off;
 
     const int t = threadIdx.x;
-    const int lane = t & 63, wave = t >> 6;
+    // a fixup launch runs one wave per workgroup; it stands in for wave blockIdx.x % 8 of the tile's workgroup
+    const int lane = t & 63, wave = fixup ? (int)(blockIdx.x & 7) : t >> 6;
     const int lb = lane & (MB - 1), hq = lane / MB;  // row inside an MFMA block, contraction chunk inside a step
     const int wave_m0 = (wave / kWavesN) * WM, wave_n0 = (wave % kWavesN) * WN;
 
@@ -539,7 +570,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     auto phase_reads = [&](int ph) { return PF * kPReadsPerFrag + (phase_reads_q(ph) ? TJ * kQReadsPerFrag : 0); };
 
     const int n_slabs = (K + BKE - 1) / BKE;
-    const bool aux_pref = kAuxPrefetch && n_slabs >= 2;  // both tail slabs exist
+    const bool aux_pref = kAuxPrefetch && n_slabs >= 2 && split_part < 0 && !fixup;  // both tail slabs exist
     u32x4 pf[2][PF], qf[2][TJ];
     // the fragments of phase ph, in the order its MFMAs (x outer, y inner) first need them
     auto read_phase = [&](int ph, const unsigned char *sp, const unsigned char *sq) {
@@ -650,7 +681,52 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
         if (want_bias) run_loop(std::true_type{});
         else run_loop(std::false_type{});
     } else {
-        run_loop(std::false_type{});
+        if (!fixup) run_loop(std::false_type{});
+    }
+
+    // Split tail tiles.  Part p of tail tile i keeps its accumulators in
+    // split_ws[(i * k_split + p) * BM * BN ...] as [float4 index j][thread], j running over
+    // (block column, block row, quarter of the block's registers): every store and load
+    // instruction of a wave covers 1 KiB of consecutive memory.
+    if constexpr (RAGGED == kRaggedRows) {
+        constexpr int kVecPerBlk = kAccRegs / 4;
+        constexpr int64_t kTileVecs = (int64_t)BM * BN / 4;
+        if (split_part >= 0) {
+            f32x4 *dst = (f32x4 *)prm.split_ws + ((int64_t)tail_index * prm.k_split + split_part) * kTileVecs + t;
+#pragma unroll
+            for (int x = 0; x < TI; ++x)
+#pragma unroll
+                for (int y = 0; y < TJ; ++y)
+#pragma unroll
+                    for (int v = 0; v < kVecPerBlk; ++v) {
+                        const int j = (x * TJ + y) * kVecPerBlk + v;
+                        f32x4 val;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) val[i] = acc[x][y][4 * v + i];
+                        __builtin_nontemporal_store(val, dst + (int64_t)j * kThreads);
+                    }
+            return;
+        }
+        if (fixup) {
+            // the parts have been added up into part 0 by split_reduce_kernel; loads go out eight at a time
+            const f32x4 *src = (const f32x4 *)prm.split_ws + (int64_t)tail_index * prm.k_split * kTileVecs + wave * 64 + lane;
+            constexpr int kVecs = TI * TJ * kVecPerBlk, kBatch = 8;
+            static_assert(kVecs % kBatch == 0, "accumulator vectors are loaded in batches of eight");
+#pragma unroll
+            for (int j0 = 0; j0 < kVecs; j0 += kBatch) {
+                f32x4 val[kBatch];
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i) val[i] = __builtin_nontemporal_load(src + (int64_t)(j0 + i) * kThreads);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i) {
+                    const int j = j0 + i, blk = j / kVecPerBlk, v = j % kVecPerBlk;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) acc[blk / TJ][blk % TJ][4 * v + c] = val[i][c];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
     }
 
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
@@ -691,7 +767,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     constexpr int CPP = 256 / (int)sizeof(T);    // C columns per pass through the staging area
     constexpr int XPP = CPP / MB;                // MFMA block columns per pass
     constexpr int NPASS = WN / CPP;
-    unsigned char *stg = smem + wave * (WM * kStgRow);
+    unsigned char *stg = smem + (fixup ? 0 : wave) * (WM * kStgRow);
     const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride + n0 : nullptr;
     T *aux = prm.aux ? (T *)prm.aux + aux_off : nullptr;
     const bool accumulate = (RAGGED == kRaggedK) && prm.accumulate_first && ei == 0;
@@ -848,33 +924,116 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
+// Adds the k_split partial accumulator tiles of every split tail tile into the first of them,
+// in ascending part order (a fixed order: the sum does not depend on scheduling).  One thread
+// per 16 bytes of a tile, all of a thread's loads issued before the first add.
+template <int kMaxSplit>
+__global__ __launch_bounds__(256) void split_reduce_kernel(float *ws, int k_split, int64_t tile_vecs, int64_t total_vecs) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total_vecs) return;
+    const int64_t tile = i / tile_vecs, v = i - tile * tile_vecs;
+    f32x4 *base = (f32x4 *)ws + tile * k_split * tile_vecs + v;
+    f32x4 part[kMaxSplit];
+#pragma unroll
+    for (int p = 0; p < kMaxSplit; ++p)
+        if (p < k_split) part[p] = __builtin_nontemporal_load(base + (int64_t)p * tile_vecs);
+    f32x4 sum = part[0];
+#pragma unroll
+    for (int p = 1; p < kMaxSplit; ++p)
+        if (p < k_split) sum += part[p];
+    base[0] = sum;
+}
+constexpr int kMaxSplit = 8;
+
+// Host-side services of grouped_gemm.hip: compute units of the current device, and a per-stream
+// buffer for the partial accumulators of split tail tiles (allocated on first use, kept until
+// the process ends; NULL when the allocation fails, in which case nothing is split).
+int device_compute_units();
+float *split_workspace(hipStream_t stream, size_t bytes);
+
+// How the tiles of a ragged-rows launch are spread over the chip.  One workgroup occupies a
+// compute unit, so `total` tiles run in total / cus rounds and a last, partial round costs as
+// much as a whole one.  When that last round fills at most half the chip, its tiles are split
+// along the contraction into k_split parts (as many as fit the idle units, at most 8, at
+// least 16 slabs each).
+struct TailSplit {
+    int main_tiles, k_split, split_slabs;
+};
+inline TailSplit plan_tail_split(int total, int n_slabs, int cus) {
+    TailSplit p{total, 1, n_slabs};
+    const int tail = total % cus;
+    if (tail == 0 || tail * 2 > cus) return p;
+    int f = std::min(std::min(kMaxSplit, cus / tail), n_slabs / 16);
+    if (f < 2) return p;
+    p.split_slabs = (n_slabs + f - 1) / f;
+    p.k_split = (n_slabs + p.split_slabs - 1) / p.split_slabs;  // no empty part
+    p.main_tiles = total - tail;
+    return p;
+}
+
 template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI>
 int launch_tiles(GemmParams &prm, hipStream_t stream) {
     // three P and two Q slab buffers, or the epilogue's staging area (one [rows][256 B + 16 B] block per wave)
     constexpr int smem_loop = (3 * BN + 2 * BM) * kSlabBytes;
-    constexpr int smem_epi = kWavesM * kWavesN * (BM / kWavesM) * (256 + 16);
+    constexpr int smem_wave_epi = (BM / kWavesM) * (256 + 16);
+    constexpr int smem_epi = kWavesM * kWavesN * smem_wave_epi;
     constexpr int smem = smem_loop > smem_epi ? smem_loop : smem_epi;
-    // the opt-in to more than 64 KiB of dynamic LDS is per device
-    static bool configured[16] = {};
+    // the opt-in to more than 64 KiB of dynamic LDS is per device (and per kernel instantiation)
+    static std::once_flag configured[16];
     auto kern = grouped_gemm_kernel<T, BM, BN, PS, QS, RG, EPI>;
     int dev = 0;
     FMOE_HIP_CHECK(hipGetDevice(&dev));
     FMOE_REQUIRE(dev >= 0 && dev < 16, "device index %d out of range", dev);
-    if (!configured[dev]) {
-        FMOE_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured[dev] = true;
-    }
+    hipError_t attr_err = hipSuccess;
+    std::call_once(configured[dev], [&]() {
+        attr_err = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    });
+    FMOE_HIP_CHECK(attr_err);
     if (prm.total_tiles <= 0) return FMOE_OK;
-    // ragged rows: the tiles rounded up to a multiple of 8; ragged K: 8 XCDs x experts x an
-    // eighth (rounded up) of one expert's tiles -- the kernel drops the surplus workgroups
-    const int64_t grid64 = (RG == kRaggedRows)
-                               ? ((int64_t)prm.total_tiles + 7) / 8 * 8
-                               : (int64_t)8 * prm.tab.n * (((int64_t)prm.tiles_m * prm.tiles_n + 7) / 8);
+    prm.main_tiles = prm.total_tiles;
+    prm.k_split = 1;
+    prm.split_slabs = 0;
+    prm.fixup = 0;
+    prm.split_ws = nullptr;
+    int64_t grid64;
+    if (RG == kRaggedRows) {
+        constexpr int BKE = kSlabBytes / (int)sizeof(T);
+        const int n_slabs = (prm.k_extent + BKE - 1) / BKE;
+        const TailSplit ts = plan_tail_split(prm.total_tiles, n_slabs, device_compute_units());
+        if (ts.k_split > 1) {
+            const int tail = prm.total_tiles - ts.main_tiles;
+            float *ws = split_workspace(stream, (size_t)tail * ts.k_split * BM * BN * sizeof(float));
+            if (ws != nullptr) {
+                prm.split_ws = ws;
+                prm.main_tiles = ts.main_tiles;
+                prm.k_split = ts.k_split;
+                prm.split_slabs = ts.split_slabs;
+            }
+        }
+        // whole tiles rounded up to a multiple of 8 (one range per XCD), then the parts of the tail tiles
+        grid64 = ((int64_t)prm.main_tiles + 7) / 8 * 8 + (int64_t)(prm.total_tiles - prm.main_tiles) * prm.k_split;
+    } else {
+        // 8 XCDs x experts x an eighth (rounded up) of one expert's tiles -- the kernel drops the surplus workgroups
+        grid64 = (int64_t)8 * prm.tab.n * (((int64_t)prm.tiles_m * prm.tiles_n + 7) / 8);
+    }
     if (grid64 > (int64_t)INT32_MAX) return fail(FMOE_ELIMIT, "grouped GEMM: grid of %lld workgroups", (long long)grid64);
     const int grid = (int)grid64;
     ProfileScope prof(prm.profile_class, prm.profile_work, stream);
     kern<<<grid, kThreads, smem, stream>>>(prm);
     FMOE_LAUNCH_CHECK();
+    if (prm.k_split > 1) {
+        // the parts are complete when the first launch has ended: add them up, then run the epilogue,
+        // one wave (its share of the tile) per workgroup
+        const int tail = prm.total_tiles - prm.main_tiles;
+        const int64_t tile_vecs = (int64_t)BM * BN / 4, total_vecs = tile_vecs * tail;
+        split_reduce_kernel<kMaxSplit><<<(unsigned)((total_vecs + 255) / 256), 256, 0, stream>>>(prm.split_ws, prm.k_split, tile_vecs, total_vecs);
+        FMOE_LAUNCH_CHECK();
+        prm.fixup = 1;
+        kern<<<(prm.total_tiles - prm.main_tiles) * kWavesM * kWavesN, 64, smem_wave_epi, stream>>>(prm);
+        FMOE_LAUNCH_CHECK();
+        prm.fixup = 0;
+    }
     return FMOE_OK;
 }
 

@@ -21,6 +21,8 @@
 
 #include <algorithm>
 #include <initializer_list>
+#include <mutex>
+#include <vector>
 
 namespace fmoe {
 using namespace gemm;
@@ -237,6 +239,16 @@ int launch_plain(GemmParams &prm, int epi, hipStream_t stream) {
 
 enum Product { kFwd = 0, kDgrad = 1, kWgrad = 2 };
 
+struct SplitBuffer {
+    int device;
+    hipStream_t stream;
+    float *ptr;
+    size_t bytes;
+};
+std::mutex g_split_mutex;
+std::vector<SplitBuffer> g_split_buffers;
+int g_compute_units[16] = {};
+
 template <int PRODUCT>
 int dispatch(GemmParams &prm, int dtype, int epi, bool fast, hipStream_t stream) {
     constexpr int RG = PRODUCT == kWgrad ? kRaggedK : kRaggedRows;
@@ -274,6 +286,45 @@ bool is_fast(int dtype, std::initializer_list<const void *> ptrs, std::initializ
 }
 
 }  // namespace
+
+namespace gemm {
+
+int device_compute_units() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 256;
+    std::lock_guard<std::mutex> lock(g_split_mutex);
+    if (g_compute_units[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        g_compute_units[dev] = n;
+    }
+    return g_compute_units[dev];
+}
+
+// One buffer per (device, stream): launches on one stream run in order, so they can share it;
+// launches on different streams may overlap and get their own.
+float *split_workspace(hipStream_t stream, size_t bytes) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_split_mutex);
+    for (SplitBuffer &b : g_split_buffers) {
+        if (b.device != dev || b.stream != stream) continue;
+        return b.bytes >= bytes ? b.ptr : nullptr;
+    }
+    if (g_split_buffers.size() >= 32) return nullptr;  // a process that keeps creating streams: stop splitting
+    // a split launch never has more parts than compute units, each a tile of at most 256 x 256
+    // floats: sized for that once, the buffer fits every later request
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    size_t want = (size_t)cus * 256 * 256 * sizeof(float);
+    if (want < bytes) want = bytes;
+    float *ptr = nullptr;
+    if (hipMalloc((void **)&ptr, want) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    g_split_buffers.push_back(SplitBuffer{dev, stream, ptr, want});
+    return ptr;
+}
+
+}  // namespace gemm
 
 int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
                            int64_t row_hi, hipStream_t stream) {
@@ -387,6 +438,18 @@ int grouped_bias_grad(const void *gy, void *gb, int64_t out_feat, int dtype, con
 }  // namespace fmoe
 
 using namespace fmoe;
+
+extern "C" int fmoe_gemm_tail_plan(int64_t total_tiles, int64_t contraction_slabs, int compute_units, int64_t *plan_host) {
+    FMOE_REQUIRE(plan_host && total_tiles >= 0 && total_tiles < (int64_t)INT32_MAX && contraction_slabs >= 0 &&
+                     contraction_slabs < (int64_t)INT32_MAX && compute_units >= 0,
+                 "fmoe_gemm_tail_plan: bad argument");
+    const gemm::TailSplit ts = gemm::plan_tail_split((int)total_tiles, (int)contraction_slabs,
+                                                     compute_units > 0 ? compute_units : gemm::device_compute_units());
+    plan_host[0] = ts.main_tiles;
+    plan_host[1] = ts.k_split;
+    plan_host[2] = ts.split_slabs;
+    return FMOE_OK;
+}
 
 extern "C" int fmoe_linear_forward(const void *x, const void *w, const void *bias, void *y,
                                    const int64_t *expert_count_host, int64_t n_expert, int64_t in_feat,

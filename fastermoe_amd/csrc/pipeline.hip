@@ -106,23 +106,59 @@ int check_common(const char *who, const fmoe_mlp_params *p, const int64_t *count
     return FMOE_OK;
 }
 
-// Chunk c covers the sorted rows [bounds[c], bounds[c+1]).  The split is even, except
-// that a boundary moves to the nearest expert boundary when one lies within a quarter
-// of a chunk: an expert that is not cut needs no partial row tile and its weight
-// gradient is produced by one chunk instead of being accumulated over two.
-void chunk_bounds(const int64_t *counts, int64_t n_expert, int64_t n_rows, int n_chunks, int64_t *bounds) {
+constexpr int kTileRows = 256;  // row-tile height of the grouped GEMM (a 128-row launch tiles the same edges)
+
+int64_t gcd64(int64_t a, int64_t b) { return b == 0 ? a : gcd64(b, a % b); }
+
+// Row position at which the first `tiles` row tiles of the expert-sorted order end (an
+// expert's rows are tiled from the expert's own first row, its last tile may be partial).
+int64_t rows_of_tiles(const int64_t *counts, int64_t n_expert, int64_t tiles) {
+    int64_t start = 0;
+    for (int64_t e = 0; e < n_expert && tiles > 0; ++e) {
+        const int64_t t = ceil_div(counts[e], kTileRows);
+        if (tiles < t) return start + tiles * kTileRows;
+        tiles -= t;
+        start += counts[e];
+    }
+    return start;
+}
+
+// Chunk c covers the sorted rows [bounds[c], bounds[c+1]).  Every bound lies on the edge of a
+// row tile of the grouped GEMM, so cutting an expert's rows adds no partial tile.  A chunk of
+// t row tiles launches t * ceil(width / 256) workgroups per product, and the chip runs them
+// `cus` at a time, a last partial round costing as much as a whole one: when the chunks are long
+// enough, all but the last get a tile count that makes both products' launches (output widths
+// d_model and d_hidden) whole numbers of rounds, and the last one takes what is left.
+void chunk_bounds(const int64_t *counts, int64_t n_expert, int64_t n_rows, int n_chunks, int64_t d_model,
+                  int64_t d_hidden, int cus, int64_t *bounds) {
+    int64_t tiles = 0;
+    for (int64_t e = 0; e < n_expert; ++e) tiles += ceil_div(counts[e], kTileRows);
+    // smallest tile count whose launches fill whole rounds for both widths
+    const int64_t wd = ceil_div(d_model, 256), wh = ceil_div(d_hidden, 256);
+    const int64_t ud = cus / gcd64(cus, wd), uh = cus / gcd64(cus, wh);
+    const int64_t unit = ud / gcd64(ud, uh) * uh;
+    int64_t per = -1;  // row tiles of every chunk but the last; -1: split the tiles evenly
+    if (unit * n_chunks <= tiles) {
+        per = (tiles + (int64_t)n_chunks * unit / 2) / ((int64_t)n_chunks * unit) * unit;  // nearest multiple to tiles / n_chunks
+        if (per * (n_chunks - 1) >= tiles) per -= unit;
+    }
     bounds[0] = 0;
     for (int c = 1; c < n_chunks; ++c) {
-        const int64_t target = n_rows * c / n_chunks;
-        int64_t best = -1, start = 0;
-        for (int64_t e = 0; e <= n_expert; ++e) {
-            if (best < 0 || llabs(start - target) < llabs(best - target)) best = start;
-            if (e < n_expert) start += counts[e];
-        }
-        int64_t b = (llabs(best - target) * 4 * n_chunks <= n_rows) ? best : target;
+        const int64_t t = per > 0 ? per * c : tiles * c / n_chunks;
+        const int64_t b = rows_of_tiles(counts, n_expert, t);
         bounds[c] = b < bounds[c - 1] ? bounds[c - 1] : b;
     }
     bounds[n_chunks] = n_rows;
+}
+
+int compute_units_or_default() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 256; }
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    return n;
 }
 
 inline const char *at(const void *base, int64_t row, int64_t row_elems, int dtype) {
@@ -138,16 +174,18 @@ inline char *at(void *base, int64_t row, int64_t row_elems, int dtype) {
 using namespace fmoe;
 
 extern "C" int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert, int n_chunks,
-                                       int64_t *bounds_host) {
+                                       int64_t d_model, int64_t d_hidden, int compute_units, int64_t *bounds_host) {
     FMOE_REQUIRE(expert_count_host && bounds_host && n_expert >= 1, "fmoe_fused_chunk_bounds: bad argument");
     FMOE_REQUIRE(n_chunks >= 1 && n_chunks <= kMaxChunks, "fmoe_fused_chunk_bounds: n_chunks=%d (1..%d)", n_chunks,
                  kMaxChunks);
+    FMOE_REQUIRE(d_model >= 1 && d_hidden >= 1 && compute_units >= 0, "fmoe_fused_chunk_bounds: bad sizes");
     int64_t rows = 0;
     for (int64_t e = 0; e < n_expert; ++e) {
         FMOE_REQUIRE(expert_count_host[e] >= 0, "fmoe_fused_chunk_bounds: negative expert count");
         rows += expert_count_host[e];
     }
-    chunk_bounds(expert_count_host, n_expert, rows, n_chunks, bounds_host);
+    chunk_bounds(expert_count_host, n_expert, rows, n_chunks, d_model, d_hidden,
+                 compute_units > 0 ? compute_units : compute_units_or_default(), bounds_host);
     return FMOE_OK;
 }
 
@@ -170,7 +208,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     if (int rc = get_lanes(&l)) return rc;
     if (int rc = fork_lanes(l, caller)) return rc;
     int64_t bounds[kMaxChunks + 1];
-    chunk_bounds(expert_count_host, E, n_rows, n_chunks, bounds);
+    chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, compute_units_or_default(), bounds);
 
     // dropped slots become zero rows; independent of everything else
     if (out && n_rows < n_slots)
@@ -227,7 +265,7 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     if (int rc = get_lanes(&l)) return rc;
     if (int rc = fork_lanes(l, caller)) return rc;
     int64_t bounds[kMaxChunks + 1];
-    chunk_bounds(expert_count_host, E, n_rows, n_chunks, bounds);
+    chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, compute_units_or_default(), bounds);
 
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
@@ -238,30 +276,33 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
                 return rc;
         FMOE_HIP_CHECK(hipEventRecord(l->in_ready[c], l->in));
     }
-    // The last chunk (even when it is empty) also zero-fills the experts without rows.
-    int last = n_chunks - 1;
+    // Per chunk, only the products a later stage waits for: the two data gradients.
+    const bool has_act = p->activation != FMOE_ACT_NONE;
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
-        const bool is_last = c == last;
-        if (hi == lo && !is_last) continue;
-        if (hi > lo) FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
-        // second linear: g_mid = (g_out . W2) * act'(pre);  gW2 (+)= g_out^T . mid;  gb2 (+)= colsum(g_out) (inside the weight-gradient kernel)
-        const bool has_act = p->activation != FMOE_ACT_NONE;
+        if (hi == lo) continue;
+        FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
+        // g_mid = (g_out . W2) * act'(pre);  g_in = g_mid . W1
         LinearDgradArgs d2{g_out, p->w2, g_mid, has_act ? buf_pre : nullptr, h, d, dt,
                            has_act ? kEpiDAct : kEpiStore, p->activation};
         if (int rc = grouped_linear_dgrad(d2, expert_count_host, E, lo, hi, l->compute)) return rc;
-        LinearWgradArgs w2{g_out, buf_mid, grad_w2, grad_b2, h, d, dt};
-        if (int rc = grouped_linear_wgrad(w2, expert_count_host, E, lo, hi, is_last, l->compute)) return rc;
-        // first linear: g_in = g_mid . W1;  gW1 (+)= g_mid^T . buf_in;  gb1 (+)= colsum(g_mid) (likewise)
         LinearDgradArgs d1{g_mid, p->w1, g_in, nullptr, d, h, dt, kEpiStore, FMOE_ACT_NONE};
         if (int rc = grouped_linear_dgrad(d1, expert_count_host, E, lo, hi, l->compute)) return rc;
-        LinearWgradArgs w1{g_mid, buf_in, grad_w1, grad_b1, d, h, dt};
-        if (int rc = grouped_linear_wgrad(w1, expert_count_host, E, lo, hi, is_last, l->compute)) return rc;
     }
-    if (int rc = join_lanes(l, caller)) return rc;
-    // grad_inp[t] = sum of the token's k expert-row gradients (rows of different
-    // chunks, so this runs once, after all of them)
+    // grad_inp[t] = sum of the token's k expert-row gradients (rows of different chunks, so
+    // this runs once, after all of them) -- on the permute-out lane, beside the weight gradients
+    FMOE_HIP_CHECK(hipEventRecord(l->out_ready[0], l->compute));
+    FMOE_HIP_CHECK(hipStreamWaitEvent(l->out, l->out_ready[0], 0));
     if (n_tokens > 0)
-        if (int rc = fmoe_reduce_slots(g_in, slot_to_row, grad_inp, n_tokens, top_k, n_rows, d, dt, caller)) return rc;
-    return FMOE_OK;
+        if (int rc = fmoe_reduce_slots(g_in, slot_to_row, grad_inp, n_tokens, top_k, n_rows, d, dt, l->out)) return rc;
+    // The weight gradients contract over an expert's rows, all of which exist now: one launch
+    // per linear over all rows, so an expert's gradient is accumulated in fp32 from start to end
+    // and rounded once, whatever the chunking (experts without rows are zero-filled):
+    // gW2 = g_out^T . mid, gb2 = colsum(g_out);  gW1 = g_mid^T . buf_in, gb1 = colsum(g_mid)
+    // (the bias gradients come out of the weight-gradient kernel's first column tiles).
+    LinearWgradArgs w2{g_out, buf_mid, grad_w2, grad_b2, h, d, dt};
+    if (int rc = grouped_linear_wgrad(w2, expert_count_host, E, 0, n_rows, true, l->compute)) return rc;
+    LinearWgradArgs w1{g_mid, buf_in, grad_w1, grad_b1, d, h, dt};
+    if (int rc = grouped_linear_wgrad(w1, expert_count_host, E, 0, n_rows, true, l->compute)) return rc;
+    return join_lanes(l, caller);
 }

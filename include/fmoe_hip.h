@@ -205,6 +205,18 @@ int fmoe_linear_backward(const void *grad_y, const void *x, const void *w,
                          int64_t in_feat, int64_t out_feat, int dtype,
                          void *stream);
 
+/* How a forward / data-grad launch of `total_tiles` output tiles (256 x 256, or
+ * 128 x 256 for small launches) with `contraction_slabs` slabs of 128
+ * contraction bytes is spread over `compute_units` (0: the current device's):
+ * plan_host[0] tiles are computed whole, one workgroup each; the rest -- the
+ * last, partial round of the chip when it fills at most half of it -- are
+ * split along the contraction into plan_host[1] parts of plan_host[2] slabs,
+ * whose fp32 partial sums are added in ascending order before the epilogue.
+ * Host only.  No counterpart in the reference (its per-expert cuBLAS calls,
+ * cuda/parallel_linear.cuh:55-88, leave this to the library). */
+int fmoe_gemm_tail_plan(int64_t total_tiles, int64_t contraction_slabs,
+                        int compute_units, int64_t *plan_host);
+
 /* ---- fused expert MLP, chunked pipeline at world_size 1 ----------------- */
 
 typedef struct fmoe_mlp_params {
@@ -219,11 +231,15 @@ typedef struct fmoe_mlp_params {
 
 /* Row bounds of the pipeline's chunks: chunk c covers the expert-sorted rows
  * [bounds_host[c], bounds_host[c+1]), bounds_host has n_chunks + 1 entries.
- * The split is even except that a bound moves to an expert boundary lying
- * within a quarter chunk of it.  Host only, no GPU work.  Plays the part of
- * the worker-group stepping of cuda/fused_compute.cuh:276-280. */
+ * Every bound lies on a row-tile edge of the grouped GEMM (256 rows, counted
+ * from each expert's first row), and when the chunks are long enough all but
+ * the last hold a tile count whose launches, for output widths d_model and
+ * d_hidden, are whole rounds of `compute_units` workgroups (0: the current
+ * device's count, 256 without a device).  Host only, no GPU work.  Plays the
+ * part of the worker-group stepping of cuda/fused_compute.cuh:276-280. */
 int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert,
-                            int n_chunks, int64_t *bounds_host);
+                            int n_chunks, int64_t d_model, int64_t d_hidden,
+                            int compute_units, int64_t *bounds_host);
 
 /* Forward of scatter -> Linear -> act -> Linear -> gather over `n_chunks`
  * contiguous chunks of the expert-sorted rows, chunk c+1's scatter and chunk
@@ -254,8 +270,10 @@ int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
  * (e.g. with fmoe_gather_combine_backward).
  * Scratch (caller-allocated): g_out [n_rows,d_model], g_mid [n_rows,d_hidden],
  * g_in [n_rows,d_model].  Results: grad_inp [n_tokens,d_model], grad_w1/2,
- * grad_b1/2 (bias grads may be NULL).  Weight grads of an expert split across
- * chunks accumulate chunk by chunk (cuda/fused_compute.cuh:123: beta_weight).
+ * grad_b1/2 (bias grads may be NULL).  The data gradients run chunk by chunk;
+ * the weight gradients run once over all rows after the last chunk, so an
+ * expert's gradient is rounded once however the rows are chunked (the
+ * reference accumulates them step by step, cuda/fused_compute.cuh:123).
  * Replaces fmoe_cuda_fused_backward_impl at one worker,
  * cuda/fused_compute.cuh:391-542 (fmoe_cuda.fused_backward). */
 int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *grad_out,

@@ -17,7 +17,10 @@ Gradients come from torch autograd on this forward, as in the reference's tests
 Pinning (tests/test_oracle.py): against a dense one-hot formulation that shares
 no code with the masked loop (einsum over all experts, then select), against a
 hand-worked 2-token case, and against ``torch.nn.Linear``/``nn.Sequential`` when
-there is a single expert.
+there is a single expert.  ``moe_mlp_forward_backward_per_expert`` (the same
+forward with the textbook backward written out, one expert at a time, for shapes
+whose float64 autograd graph would not fit in memory) is pinned against the
+autograd version on small shapes.
 """
 import time
 
@@ -71,6 +74,61 @@ def moe_mlp_forward_backward(inp, gate_idx, gate_score, w1, b1, w2, b2, activati
     g = lambda t: None if t is None else t.grad
     return {"out": out.detach(), "grad_inp": x.grad, "grad_w1": W1.grad, "grad_b1": g(B1),
             "grad_w2": W2.grad, "grad_b2": g(B2)}
+
+
+def moe_mlp_forward_backward_per_expert(inp, gate_idx, gate_score, w1, b1, w2, b2, activation, top_k,
+                                        grad_out=None, grad_dtype=torch.float64):
+    """Same results as ``moe_mlp_forward_backward`` (float64, ``out.mean()`` as the loss
+    unless ``grad_out`` [N,d] is given), computed one expert at a time with the backward of
+    ``Linear -> activation -> Linear`` and of the score-weighted sum written out, so that
+    only one expert's weights are held in float64 at a time.  ``activation``: "gelu"
+    (exact) or "relu".  Gate scores get no gradient here.  The weight gradients are stored
+    in ``grad_dtype`` (float32 halves the memory of very large layers)."""
+    f64 = torch.float64
+    x = inp.detach().to("cpu", f64)
+    n, d = x.shape
+    idx = gate_idx.detach().cpu().long().reshape(-1)
+    score = gate_score.detach().to("cpu", f64).reshape(-1)
+    g_out = torch.full((n, d), 1.0 / (n * d), dtype=f64) if grad_out is None else grad_out.detach().to("cpu", f64)
+    out = torch.zeros(n, d, dtype=f64)
+    res = {"out": out, "grad_inp": torch.zeros(n, d, dtype=f64),
+           "grad_w1": torch.zeros(w1.shape, dtype=grad_dtype), "grad_w2": torch.zeros(w2.shape, dtype=grad_dtype),
+           "grad_b1": None if b1 is None else torch.zeros(b1.shape, dtype=f64),
+           "grad_b2": None if b2 is None else torch.zeros(b2.shape, dtype=f64)}
+    for e in range(w1.shape[0]):
+        slots = torch.nonzero(idx == e).reshape(-1)
+        if slots.numel() == 0:
+            continue
+        tok = slots // top_k
+        W1, W2 = w1[e].detach().to("cpu", f64), w2[e].detach().to("cpu", f64)
+        xe = x[tok]
+        pre = xe @ W1.t()
+        if b1 is not None:
+            pre = pre + b1[e].detach().to("cpu", f64)
+        if activation == "gelu":
+            cdf = 0.5 * (1.0 + torch.erf(pre / 2.0 ** 0.5))
+            mid = pre * cdf
+            dact = cdf + pre * torch.exp(-0.5 * pre * pre) / (2.0 * torch.pi) ** 0.5
+        elif activation == "relu":
+            mid = pre.clamp_min(0.0)
+            dact = (pre > 0).to(f64)
+        else:
+            raise ValueError(activation)
+        y = mid @ W2.t()
+        if b2 is not None:
+            y = y + b2[e].detach().to("cpu", f64)
+        sc = score[slots].unsqueeze(1)
+        out.index_add_(0, tok, sc * y)
+        gy = sc * g_out[tok]
+        res["grad_w2"][e] = gy.t() @ mid
+        g_pre = (gy @ W2) * dact
+        res["grad_w1"][e] = g_pre.t() @ xe
+        if b2 is not None:
+            res["grad_b2"][e] = gy.sum(0)
+        if b1 is not None:
+            res["grad_b1"][e] = g_pre.sum(0)
+        res["grad_inp"].index_add_(0, tok, g_pre @ W1)
+    return res
 
 
 def per_expert_linear(inp_sorted, counts, weight, bias):

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in fmoe_hip.h but not exported"
     assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header disagree"
-    assert lib.fmoe_abi_version() == 1
+    assert lib.fmoe_abi_version() == 2
 
 
 def test_ctypes_signatures_match_the_header():
@@ -157,32 +157,79 @@ def test_activation_codes():
 
 
 def test_fused_chunk_bounds_host_logic():
-    """Chunk planning of the fused pipeline (host only): monotone, covers all rows, snaps to an
-    expert boundary within a quarter chunk, otherwise splits evenly."""
+    """Chunk planning of the fused pipeline (host only): monotone, covers all rows, every bound on a
+    row-tile edge, and -- when the chunks are long enough -- whole rounds of workgroups for both
+    output widths in every chunk but the last."""
     import ctypes
     lib = _lib.load()
 
-    def bounds(counts, n_chunks):
+    def bounds(counts, n_chunks, d=4096, h=14336, cus=256):
         c = (ctypes.c_int64 * len(counts))(*counts)
         b = (ctypes.c_int64 * (n_chunks + 1))()
-        _lib.check(lib.fmoe_fused_chunk_bounds(ctypes.cast(c, ctypes.c_void_p), len(counts), n_chunks,
+        _lib.check(lib.fmoe_fused_chunk_bounds(ctypes.cast(c, ctypes.c_void_p), len(counts), n_chunks, d, h, cus,
                                                ctypes.cast(b, ctypes.c_void_p)))
         return list(b)
 
-    # 8 nearly equal experts, 4 chunks: every bound lands on an expert boundary
+    def tiles_between(counts, lo, hi):
+        """Row tiles of 256 of the rows [lo, hi), every expert tiled from its own first row."""
+        t, start = 0, 0
+        for n in counts:
+            a, b = max(lo, start), min(hi, start + n)
+            if b > a:
+                t += -(-(b - a) // 256)
+            start += n
+        return t
+
+    def tile_edges(counts):
+        edges, start = {0}, 0
+        for n in counts:
+            edges |= {start + r for r in range(256, n, 256)} | {start + n}
+            start += n
+        return edges
+
+    # the Mixtral-like share: 8 nearly equal experts, 4 chunks -> 64 row tiles (4 and 14 whole rounds
+    # of 256 workgroups for widths 4096 and 14336) in the first three chunks, the rest in the last
     counts = [8100, 8300, 8192, 8000, 8400, 8192, 8150, 8202]
     b = bounds(counts, 4)
-    prefix = [sum(counts[:i]) for i in range(9)]
-    assert b[0] == 0 and b[-1] == sum(counts) and all(x in prefix for x in b)
-    # one huge expert: no boundary nearby, even split
-    assert bounds([1000], 4) == [0, 250, 500, 750, 1000]
-    # boundary too far from the even split stays even
-    assert bounds([100, 900], 2) == [0, 500, 1000]
-    # boundary within a quarter chunk is taken
-    assert bounds([450, 550], 2) == [0, 450, 1000]
+    assert b[0] == 0 and b[-1] == sum(counts) and all(x <= y for x, y in zip(b, b[1:]))
+    assert all(x in tile_edges(counts) for x in b)
+    per_chunk = [tiles_between(counts, lo, hi) for lo, hi in zip(b, b[1:])]
+    assert per_chunk[:3] == [64, 64, 64] and sum(per_chunk) == sum(-(-n // 256) for n in counts)
+    for t in per_chunk[:3]:
+        assert t * 16 % 256 == 0 and t * 56 % 256 == 0
+    # chunks too short for whole rounds: an even split of the row tiles, still on tile edges
+    assert bounds([1000], 4) == [0, 256, 512, 768, 1000]
+    assert bounds([100, 900], 2) == [0, 356, 1000]      # 1 + 4 tiles: bound after the second tile
+    assert bounds([512, 512], 2, d=256, h=256, cus=2) == [0, 512, 1024]
     # more chunks than rows, empty experts: still monotone and complete
     b = bounds([0, 3, 0, 0, 2], 8)
     assert b[0] == 0 and b[-1] == 5 and all(x <= y for x, y in zip(b, b[1:]))
     assert bounds([0, 0], 3) == [0, 0, 0, 0]
-    rc = lib.fmoe_fused_chunk_bounds(None, 2, 3, None)
+    rc = lib.fmoe_fused_chunk_bounds(None, 2, 3, 64, 64, 0, None)
     assert rc == -1
+
+
+def test_gemm_tail_plan_host_logic():
+    """Which tiles of a launch are split along the contraction (host only)."""
+    import ctypes
+    lib = _lib.load()
+
+    def plan(tiles, slabs, cus=256):
+        out = (ctypes.c_int64 * 3)()
+        _lib.check(lib.fmoe_gemm_tail_plan(tiles, slabs, cus, ctypes.cast(out, ctypes.c_void_p)))
+        return list(out)
+
+    assert plan(1024, 224)[:2] == [1024, 1]            # whole rounds: nothing to split
+    assert plan(1040, 224) == [1024, 8, 28]            # 16 tail tiles x 8 parts of 28 slabs
+    assert plan(1104, 224) == [1024, 3, 75]            # 80 tail tiles: 3 parts fit the idle units
+    assert plan(3640, 64) == [3584, 4, 16]             # parts keep at least 16 slabs
+    assert plan(3720, 64)[:2] == [3720, 1]             # the last round fills more than half the chip
+    assert plan(80, 8)[:2] == [80, 1]                  # contraction too short to split
+    m, f, per = plan(5, 33)
+    assert (m, f) == (0, 2) and per * f >= 33 and per * (f - 1) < 33   # no empty part
+    for tiles in range(1, 600, 7):
+        for slabs in (1, 15, 16, 31, 32, 100, 224):
+            m, f, per = plan(tiles, slabs)
+            assert 0 <= m <= tiles and 1 <= f <= 8 and (tiles - m) * f <= 256 or f == 1
+            if f > 1:
+                assert per >= 16 and per * f >= slabs and per * (f - 1) < slabs and m % 256 == 0

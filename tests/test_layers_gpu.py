@@ -15,7 +15,7 @@ from fastermoe_amd.layers import FMoE
 from fastermoe_amd.transformer import _Expert
 from oracle import moe as omoe
 from oracle import routing as orouting
-from helpers import TOL, rel_err
+from helpers import TOL, assert_close, close_stats, rel_err, zipf_experts
 
 pytestmark = pytest.mark.gpu
 
@@ -47,6 +47,39 @@ def _compare(moe, x, act, top_k, dtype, grads_of_score=False):
             continue
         assert rel_err(val, ref[name]) <= tol, (name, rel_err(val, ref[name]))
     return got
+
+
+def _compare_per_expert(moe, x, idx, score, act, top_k, tol):
+    """Layer against the one-expert-at-a-time float64 oracle (for layers whose float64 autograd graph
+    would not fit in memory): max|d| <= tol max|ref|, |d| <= tol |ref| + 3 tol rms(ref) element by
+    element, and rms(d) <= tol / 2 rms(ref); the weight gradients expert by expert, against the
+    expert's own root mean square.  The floor of three: a weight gradient is a sum over the expert's
+    rows of products that went through four roundings to the element type on the way (pre-activation,
+    activation, both gradient buffers); over the 10^7 elements of such a tensor the tail of that
+    rounding noise reaches a few percent of the root mean square.  A wrong or missing term shows in the
+    rms bound, where the noise averages out."""
+    floor = 3.0
+    x = x.clone().requires_grad_(True)
+    moe.gate.forward = lambda inp: (idx, score)
+    moe.zero_grad()
+    out = moe(x)
+    out.mean().backward()
+    e = moe.experts
+    ref = omoe.moe_mlp_forward_backward_per_expert(x, idx, score, e.htoh4.weight, e.htoh4.bias, e.h4toh.weight,
+                                                   e.h4toh.bias, act, top_k, grad_dtype=torch.float32)
+    assert_close(out, ref["out"], tol, "out", floor)
+    assert_close(x.grad, ref["grad_inp"], tol, "grad_inp", floor)
+    counts = torch.bincount(idx[idx >= 0].view(-1).cpu(), minlength=e.htoh4.weight.shape[0])
+    for name, got in (("grad_w1", e.htoh4.weight.grad), ("grad_w2", e.h4toh.weight.grad),
+                      ("grad_b1", e.htoh4.bias.grad), ("grad_b2", e.h4toh.bias.grad)):
+        scale = ref[name].abs().max().item()
+        for ex in range(got.shape[0]):
+            if counts[ex] == 0:
+                assert torch.count_nonzero(got[ex]) == 0, (name, ex)
+                continue
+            _, elem, rms = close_stats(got[ex], ref[name][ex], floor)
+            big = (got[ex].double().cpu() - ref[name][ex].double()).abs().max().item() / scale
+            assert big <= tol and elem <= tol and rms <= tol / 2, (name, ex, int(counts[ex]), big, elem, rms)
 
 
 class MyMoE(FMoE):
@@ -103,6 +136,97 @@ def test_transformer_mlp_configs(fuse, dtype, n, d, h, e, k, act, device):
         idx = torch.multinomial(p / p.sum(), n, replacement=True).view(n, 1).to(device)
         moe.gate.forward = lambda inp: (idx, torch.ones(n, 1, dtype=dtype, device=device))
     _compare(moe, x, act, k, dtype)
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+@pytest.mark.parametrize("n,d,h,e,k,routing", [
+    (1024, 2048, 8192, 64, 1, "zipf"),     # the skewed Switch-style layer at full width: Zipf(1.2) top-1, empty experts
+    (512, 2048, 1024, 256, 8, "biased"),   # the fine-grained layer at full width: 256 experts, top-8
+])
+def test_full_width_bf16_layers(fuse, n, d, h, e, k, routing, device):
+    """The many-expert configurations at their real feature sizes (only the token count is reduced),
+    bf16, forward and all gradients against the float64 oracle, normwise and element by element."""
+    torch.manual_seed(e)
+    gen = torch.Generator().manual_seed(e + 1)
+    with torch.device(device):  # 2 x 1 G weights: initialised on the GPU
+        moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe.enable_fuse = fuse
+    with torch.no_grad():
+        moe.experts.htoh4.weight.mul_((d * h) ** 0.5 * d ** -0.5)   # unit-variance activations instead of ~1e-3
+        moe.experts.h4toh.weight.mul_((d * h) ** 0.5 * h ** -0.5)
+        moe.experts.htoh4.bias.normal_(0, 0.1)
+        moe.experts.h4toh.bias.normal_(0, 0.1)
+    moe = moe.to(torch.bfloat16).to(device)
+    x = torch.randn(n, d, generator=gen).bfloat16().to(device)
+    if routing == "zipf":
+        idx = zipf_experts(n, e, 1.2, gen).view(n, 1).to(device)
+        score = torch.ones(n, 1, dtype=torch.bfloat16, device=device)
+        assert int(torch.bincount(idx.view(-1).cpu(), minlength=e).max()) > n // 10
+        assert int((torch.bincount(idx.view(-1).cpu(), minlength=e) == 0).sum()) > 0
+    else:
+        logits = torch.randn(n, e, generator=gen) + 0.5 * torch.randn(e, generator=gen)
+        val, idx = torch.topk(logits, k, dim=-1)
+        idx, score = idx.to(device), torch.softmax(val, dim=-1).bfloat16().to(device)
+    _compare_per_expert(moe, x, idx, score, "gelu", k, 2e-2)
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_gshard_shaped_bf16_layer_with_capacity_drops(fuse, device):
+    """The GShard-style top-2 layer (d 1024, h 4096, 16 experts, bf16) with a per-expert capacity of
+    ceil(1.2 N k / E) applied by the capacity kernels, so that overflow slots are dropped: the gate
+    output after limit_by_capacity goes to the layer and to the float64 oracle alike."""
+    from fastermoe_amd.gates.utils import limit_by_capacity
+    torch.manual_seed(2)
+    n, d, h, e, k = 2048, 1024, 4096, 16, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe.enable_fuse = fuse
+    with torch.no_grad():
+        moe.experts.htoh4.weight.mul_((d * h) ** 0.5 * d ** -0.5)
+        moe.experts.h4toh.weight.mul_((d * h) ** 0.5 * h ** -0.5)
+        moe.experts.htoh4.bias.normal_(0, 0.1)
+        moe.experts.h4toh.bias.normal_(0, 0.1)
+    moe = moe.to(torch.bfloat16).to(device)
+    x = torch.randn(n, d).bfloat16().to(device)
+    logits = torch.randn(n, e) + torch.linspace(-0.6, 0.6, e)      # mild imbalance: some experts overflow
+    val, top = torch.topk(logits, k, dim=-1)
+    cap = math.ceil(1.2 * n * k / e)
+    _, _, idx = limit_by_capacity(top.to(device), e, 1, cap)
+    dropped = int((idx < 0).sum())
+    assert 0 < dropped < n * k // 2
+    assert int(torch.bincount(idx[idx >= 0].view(-1), minlength=e).max()) == cap
+    _, _, want = orouting.limit_and_prune(top.numpy(), e, cap)
+    assert np.array_equal(idx.cpu().numpy(), want)
+    score = torch.softmax(val, dim=-1).bfloat16().to(device)
+    _compare_per_expert(moe, x, idx, score, "gelu", k, 2e-2)
+
+
+def test_fused_bf16_expert_split_across_chunks(device, monkeypatch):
+    """Four chunks over three experts: the chunk bounds (read back from the planner) cut at least one
+    expert's rows, so its forward and data-grad rows come from two launches; output and all gradients
+    against the float64 oracle.  The weight gradients are produced by one launch over all rows."""
+    import ctypes
+    from fastermoe_amd import _lib
+    monkeypatch.setenv("FMOE_FUSE_GRAN", "4")
+    torch.manual_seed(9)
+    n, d, h, e, k = 1500, 512, 1024, 3, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe.enable_fuse = True
+    with torch.no_grad():
+        moe.experts.htoh4.weight.mul_((d * h) ** 0.5 * d ** -0.5)
+        moe.experts.h4toh.weight.mul_((d * h) ** 0.5 * h ** -0.5)
+        moe.experts.htoh4.bias.normal_(0, 0.1)
+    moe = moe.to(torch.bfloat16).to(device)
+    x = torch.randn(n, d).bfloat16().to(device)
+    idx = torch.randint(0, e, (n, k), device=device)
+    score = torch.rand(n, k, device=device).bfloat16()
+    counts = torch.bincount(idx.view(-1).cpu(), minlength=e)
+    c = (ctypes.c_int64 * e)(*counts.tolist())
+    b = (ctypes.c_int64 * 5)()
+    _lib.check(_lib.load().fmoe_fused_chunk_bounds(ctypes.cast(c, ctypes.c_void_p), e, 4, d, h, 0,
+                                                   ctypes.cast(b, ctypes.c_void_p)))
+    edges = set(torch.cumsum(counts, 0).tolist()) | {0}
+    assert any(x not in edges for x in list(b)[1:4]), "no chunk bound cuts an expert"
+    _compare_per_expert(moe, x, idx, score, "gelu", k, 2e-2)
 
 
 @pytest.mark.parametrize("fuse", [False, True])

@@ -8,7 +8,7 @@ import torch
 from fastermoe_amd import fmoe_native
 from fastermoe_amd.functions import MOELinear
 from oracle import moe as omoe
-from helpers import TOL, ragged_counts, rel_err
+from helpers import TOL, assert_close, ragged_counts, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -149,6 +149,60 @@ def test_linearity_at_full_width(device):
     assert torch.equal(yb[:700], b[0].expand(700, h)) and torch.equal(yb[700:], b[1].expand(324, h))
     ref = (x[:700].double().cpu() @ w[0].double().cpu().t())
     assert rel_err(y1[:700], ref) <= 2e-2
+
+
+@pytest.mark.parametrize("fin,fout", [(14336, 4096), (4096, 14336)])
+def test_full_depth_bf16_forward_backward(fin, fout, device):
+    """The Mixtral-like share's feature sizes at full contraction depth, both linears: bf16 forward,
+    data-grad (contraction 4096 / 14336), weight-grad and bias-grad against the float64 oracle, on
+    ragged segments that leave partial row tiles; normwise AND element by element (|d| <= tol |ref| +
+    tol rms(ref)).  Both the forward and the data-grad launch fill less than half a round of the chip
+    after their whole rounds, so they also run the contraction-split tail with its fp32 partial sums."""
+    import ctypes
+    from fastermoe_amd import _lib
+    g = torch.Generator().manual_seed(fin // 7)
+    counts = torch.tensor([350, 0, 250])
+    rows, e = 600, 3
+    x = torch.randn(rows, fin, generator=g).bfloat16()
+    w = (torch.randn(e, fout, fin, generator=g) / fin ** 0.5).bfloat16()
+    b = torch.randn(e, fout, generator=g).bfloat16()
+    gy = torch.randn(rows, fout, generator=g).bfloat16()
+    # 128-row tiles (fewer than 512 tiles of 256): 3 + 2 row tiles; both products are split
+    plan = (ctypes.c_int64 * 3)()
+    for width, depth in ((fout, fin), (fin, fout)):
+        _lib.check(_lib.load().fmoe_gemm_tail_plan(5 * ((width + 255) // 256), (depth + 63) // 64, 256,
+                                                  ctypes.cast(plan, ctypes.c_void_p)))
+        assert plan[1] > 1
+    ref_y, ref_gx, ref_gw, ref_gb = _reference(x, counts, w, b, gy)
+    xd, wd, bd, gyd = x.to(device), w.to(device), b.to(device), gy.to(device)
+    assert_close(fmoe_native.linear_forward(xd, counts, wd, bd), ref_y, 2e-2, "forward")
+    gx, gw, gb = fmoe_native.linear_backward(gyd, xd, counts, wd, bd)
+    assert_close(gx, ref_gx, 2e-2, "data-grad")
+    assert_close(gw, ref_gw, 2e-2, "weight-grad")
+    assert_close(gb, ref_gb, 2e-2, "bias-grad")
+    assert torch.count_nonzero(gw[1]) == 0 and torch.count_nonzero(gb[1]) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_contraction_split_tail_matches_oracle(dtype, device):
+    """A launch of 2 x 3 + 1 x 3 row/column tiles whose contraction (40 slabs of bf16, 80 of fp32)
+    is split into parts: forward with bias and data-grad, with a ragged contraction tail."""
+    g = torch.Generator().manual_seed(23)
+    counts = torch.tensor([200, 100])
+    fin, fout = 2560 - 8, 2560 - 24
+    x = torch.randn(300, fin, generator=g).to(dtype)
+    w = (torch.randn(2, fout, fin, generator=g) / fin ** 0.5).to(dtype)
+    b = torch.randn(2, fout, generator=g).to(dtype)
+    gy = torch.randn(300, fout, generator=g).to(dtype)
+    ref_y, ref_gx, ref_gw, ref_gb = _reference(x, counts, w, b, gy)
+    xd, wd, bd, gyd = x.to(device), w.to(device), b.to(device), gy.to(device)
+    tol = TOL[dtype]
+    assert_close(fmoe_native.linear_forward(xd, counts, wd, bd), ref_y, tol, "forward")
+    gx, gw, gb = fmoe_native.linear_backward(gyd, xd, counts, wd, bd)
+    assert_close(gx, ref_gx, tol, "data-grad")
+    assert_close(gw, ref_gw, tol, "weight-grad")
+    # twice the same call: the partial sums are added in a fixed order, so the result is reproducible
+    assert torch.equal(fmoe_native.linear_forward(xd, counts, wd, bd), fmoe_native.linear_forward(xd, counts, wd, bd))
 
 
 def test_validation_errors(device):

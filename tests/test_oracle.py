@@ -203,3 +203,35 @@ def test_per_expert_linear_matches_masked_loop():
     owner = torch.repeat_interleave(torch.arange(4), counts)
     for r in range(9):
         assert torch.allclose(y[r], w[owner[r]] @ x[r] + b[owner[r]], rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("act", ["gelu", "relu"])
+@pytest.mark.parametrize("bias", [True, False])
+def test_per_expert_backward_matches_autograd(act, bias):
+    """The written-out backward (one expert at a time) against autograd on the masked-loop
+    forward: drops, an expert without tokens, top-3."""
+    g = torch.Generator().manual_seed(17)
+    n, d, h, e, k = 37, 12, 20, 5, 3
+    x = torch.randn(n, d, generator=g)
+    idx = torch.randint(-1, e - 1, (n, k), generator=g)     # expert e-1 gets nothing, some slots dropped
+    score = torch.rand(n, k, generator=g)
+    w1, w2 = torch.randn(e, h, d, generator=g), torch.randn(e, d, h, generator=g)
+    b1 = torch.randn(e, h, generator=g) if bias else None
+    b2 = torch.randn(e, d, generator=g) if bias else None
+    ref = omoe.moe_mlp_forward_backward(x, idx, score, w1, b1, w2, b2, act, k)
+    got = omoe.moe_mlp_forward_backward_per_expert(x, idx, score, w1, b1, w2, b2, act, k)
+    for name in ref:
+        if ref[name] is None:
+            assert got[name] is None
+        else:
+            assert torch.allclose(got[name], ref[name], rtol=1e-11, atol=1e-13), name
+    # an explicit output gradient instead of the mean
+    go = torch.randn(n, d, generator=g)
+    got = omoe.moe_mlp_forward_backward_per_expert(x, idx, score, w1, b1, w2, b2, act, k, grad_out=go)
+    xx = x.double().requires_grad_(True)
+    W1 = w1.double().requires_grad_(True)
+    out = omoe.brute_force_moe_mlp(xx, idx, score.double(), W1, None if b1 is None else b1.double(), w2.double(),
+                                   None if b2 is None else b2.double(), act, k)
+    out.backward(go.double())
+    assert torch.allclose(got["grad_inp"], xx.grad, rtol=1e-11, atol=1e-13)
+    assert torch.allclose(got["grad_w1"], W1.grad, rtol=1e-11, atol=1e-13)
