@@ -94,6 +94,123 @@ def step(layer, x, grad):
     out.backward(grad)
 
 
+def gemm_algorithmic_bytes(cfg, rows, experts_used):
+    """Bytes the six grouped products of a step must move at least: every operand read once, every
+    result written once.  Per linear (in, out): forward reads rows*in + E'*in*out and writes rows*out,
+    data-grad reads rows*out + E'*in*out and writes rows*in, weight-grad reads rows*(in + out) and
+    writes E*in*out (E' = experts that have rows)."""
+    e_bytes = 2 if cfg["dtype"] == "bf16" else 4
+    d, h = cfg["d"], cfg["h"]
+    per_linear = 3 * rows * (d + h) + (2 * experts_used + cfg["e"]) * d * h
+    return 2 * per_linear * e_bytes
+
+
+def measure(cfg, name, device, steps, warmup, profile_steps, permutes_alone):
+    """Times `steps` forward + backward steps of the layer of `cfg` (after `warmup`), then `profile_steps`
+    more with the library's per-launch HIP-event brackets switched on."""
+    import torch
+    from fastermoe_amd import _lib, fmoe_native
+    layer, x, grad = build_layer(cfg, device)
+    for _ in range(warmup):
+        step(layer, x, grad)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(layer, x, grad)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / steps * 1e3
+    tokens_per_s = cfg["n"] * steps / elapsed
+
+    # per-kernel timing: HIP events recorded by the library on the stream each kernel runs on
+    _lib.profile_enable(True)
+    _lib.profile_collect()
+    for _ in range(profile_steps):
+        step(layer, x, grad)
+    prof = _lib.profile_collect()
+    _lib.profile_enable(False)
+
+    kernels = {}
+    for kname, (launches, ms, work) in prof.items():
+        if launches == 0:
+            continue
+        is_gemm = kname.startswith("gemm")
+        rate = work / (ms * 1e-3) / (1e12 if is_gemm else 1e9)
+        kernels[kname] = {"launches_per_step": launches / profile_steps,
+                          "avg_ms": round(ms / launches, 4), "ms_per_step": round(ms / profile_steps, 4),
+                          "work_per_launch": work / launches,
+                          "achieved": round(rate, 2), "unit": "TFLOP/s" if is_gemm else "GB/s"}
+    gemm_names = [k for k in kernels if k.startswith("gemm")]
+    peak = PEAK[cfg["dtype"]]
+    gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_names)
+    gemm_flop = sum(kernels[k]["work_per_launch"] * kernels[k]["launches_per_step"] for k in gemm_names)
+
+    n, k, d = cfg["n"], cfg["k"], cfg["d"]
+    with torch.no_grad():
+        idx, _ = layer.gate(x)
+        cnt, pos_buf, s2r = fmoe_native.route(idx.contiguous(), cfg["e"])
+        cnt_cpu = cnt.cpu()
+        rows, used = int(cnt_cpu.sum()), int((cnt_cpu > 0).sum())
+    gemm_bytes = gemm_algorithmic_bytes(cfg, rows, used)
+    mfma_frac = gemm_flop / (gemm_ms * 1e-3) / 1e12 / peak
+    hbm_frac = gemm_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+    gemm_all = {"tflops": round(gemm_flop / (gemm_ms * 1e-3) / 1e12, 2), "frac_of_mfma_peak": round(mfma_frac, 4),
+                "algorithmic_gbytes_per_step": round(gemm_bytes / 1e9, 3),
+                "frac_of_hbm_peak": round(hbm_frac, 4), "bound": "mfma" if mfma_frac >= hbm_frac else "hbm",
+                "ms_per_step": round(gemm_ms, 3)}
+
+    # the roof of the GEMM class with the most time per step: the nearer of the two
+    dominant = max(gemm_names, key=lambda kk: kernels[kk]["ms_per_step"])
+    dk = kernels[dominant]
+    dom_frac_mfma = dk["achieved"] / peak
+    # bytes per launch of the dominant class: its share of the step's algorithmic bytes by product
+    e_bytes = 2 if cfg["dtype"] == "bf16" else 4
+    per = {"gemm_fwd": 2 * (rows * (cfg["d"] + cfg["h"]) + used * cfg["d"] * cfg["h"]),
+           "gemm_dgrad": 2 * (rows * (cfg["d"] + cfg["h"]) + used * cfg["d"] * cfg["h"]),
+           "gemm_wgrad": 2 * (rows * (cfg["d"] + cfg["h"]) + cfg["e"] * cfg["d"] * cfg["h"])}
+    dom_bytes_per_launch = per[dominant] * e_bytes / dk["launches_per_step"]
+    dom_frac_hbm = dom_bytes_per_launch / (dk["avg_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+    if dom_frac_mfma >= dom_frac_hbm:
+        roofline = {"kernel": "grouped_gemm_kernel (" + dominant + ")", "bound": "mfma",
+                    "achieved": round(dk["achieved"], 2), "peak": peak, "unit": "TFLOP/s",
+                    "frac": round(dom_frac_mfma, 4), "flop_per_launch": dk["work_per_launch"],
+                    "avg_launch_ms": dk["avg_ms"], "frac_of_hbm_peak": round(dom_frac_hbm, 4)}
+    else:
+        roofline = {"kernel": "grouped_gemm_kernel (" + dominant + ")", "bound": "hbm",
+                    "achieved": round(dom_bytes_per_launch / (dk["avg_ms"] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": round(dom_frac_hbm, 4), "bytes_per_launch": dom_bytes_per_launch,
+                    "avg_launch_ms": dk["avg_ms"], "frac_of_mfma_peak": round(dom_frac_mfma, 4)}
+    roofline["traffic"] = TRAFFIC_BYTES.get(name, {}).get(dominant) if cfg["fuse"] else None
+
+    permute_alone = None
+    if permutes_alone:
+        # the row permutes alone (inside the fused pipeline they share the chip with the GEMMs)
+        with torch.no_grad():
+            pos = pos_buf[:rows]
+            tok = pos // k
+            _lib.profile_enable(True)
+            _lib.profile_collect()
+            for _ in range(10):
+                buf = fmoe_native.gather_rows(x.detach(), tok)            # local scatter
+                fmoe_native.gather_rows(buf, s2r, n * k)                   # local gather (copy)
+            gather_alone = _lib.profile_collect()["gather_rows"]
+            for _ in range(10):
+                fmoe_native.reduce_slots(buf, s2r, n, k)                   # backward of the scatter
+            reduce_alone = _lib.profile_collect()["reduce_slots"]
+            _lib.profile_enable(False)
+        permute_alone = {
+            "gather_rows": {"GB/s": round(gather_alone[2] / gather_alone[1] / 1e6, 1),
+                            "frac_of_hbm_peak": round(gather_alone[2] / gather_alone[1] / 1e6 / HBM_PEAK_GBS, 4)},
+            "reduce_slots": {"GB/s": round(reduce_alone[2] / reduce_alone[1] / 1e6, 1),
+                             "frac_of_hbm_peak": round(reduce_alone[2] / reduce_alone[1] / 1e6 / HBM_PEAK_GBS, 4)},
+        }
+        del buf
+    del layer, x, grad
+    torch.cuda.empty_cache()
+    return {"ms_per_step": round(ms_per_step, 3), "tokens_per_s": round(tokens_per_s, 1), "kernels": kernels,
+            "gemm_all": gemm_all, "roofline": roofline, "permute_alone": permute_alone}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -101,6 +218,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="config4", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", dest="other_configs", action="store_false",
+                    help="skip the short runs of configurations 1, 2, 3 and 5 that follow the headline workload")
     ap.add_argument("--profile-steps", type=int, default=3)
     ap.add_argument("--fuse", choices=["auto", "on", "off"], default="auto",
                     help="override the configuration's choice of the fused pipeline")
@@ -168,91 +287,37 @@ def main():
             out["vendor_library_" + name] = round(flop / timed(lambda: torch.nn.functional.linear(xx, ww[0])) / 1e9, 1)
         print(json.dumps(out))
         return
-    layer, x, grad = build_layer(cfg, device)
-
-    for _ in range(args.warmup):
-        step(layer, x, grad)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(layer, x, grad)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    tokens_per_s = cfg["n"] * args.steps / elapsed
-
-    # per-kernel timing: HIP events recorded by the library on the stream each kernel runs on
-    _lib.profile_enable(True)
-    _lib.profile_collect()
-    for _ in range(args.profile_steps):
-        step(layer, x, grad)
-    prof = _lib.profile_collect()
-    _lib.profile_enable(False)
-
-    kernels = {}
-    for name, (launches, ms, work) in prof.items():
-        if launches == 0:
-            continue
-        is_gemm = name.startswith("gemm")
-        rate = work / (ms * 1e-3) / (1e12 if is_gemm else 1e9)
-        kernels[name] = {"launches_per_step": launches / args.profile_steps,
-                         "avg_ms": ms / launches, "ms_per_step": ms / args.profile_steps,
-                         "work_per_launch": work / launches,
-                         "achieved": rate, "unit": "TFLOP/s" if is_gemm else "GB/s"}
-    gemm_names = [k for k in kernels if k.startswith("gemm")]
-    dominant = max(gemm_names, key=lambda k: kernels[k]["ms_per_step"])
-    peak = PEAK[cfg["dtype"]]
-    dk = kernels[dominant]
-    roofline = {"kernel": "grouped_gemm_kernel (" + dominant + ")", "bound": "mfma", "achieved": round(dk["achieved"], 2),
-                "peak": peak, "unit": "TFLOP/s", "frac": round(dk["achieved"] / peak, 4),
-                "flop_per_launch": dk["work_per_launch"], "avg_launch_ms": round(dk["avg_ms"], 4),
-                "traffic": TRAFFIC_BYTES.get(args.config, {}).get(dominant) if cfg["fuse"] else None}
-    # the row permutes alone (inside the fused pipeline they share the chip with the GEMMs)
-    from fastermoe_amd import fmoe_native
-    n, k, d = cfg["n"], cfg["k"], cfg["d"]
-    with torch.no_grad():
-        idx, _ = layer.gate(x)
-        cnt, pos_buf, s2r = fmoe_native.route(idx.contiguous(), cfg["e"])
-        pos = pos_buf[: int(cnt.sum())]
-        tok = pos // k
-        _lib.profile_enable(True)
-        _lib.profile_collect()
-        for _ in range(10):
-            buf = fmoe_native.gather_rows(x.detach(), tok)            # local scatter
-            fmoe_native.gather_rows(buf, s2r, n * k)                   # local gather (copy)
-        gather_alone = _lib.profile_collect()["gather_rows"]
-        for _ in range(10):
-            fmoe_native.reduce_slots(buf, s2r, n, k)                   # backward of the scatter
-        reduce_alone = _lib.profile_collect()["reduce_slots"]
-        _lib.profile_enable(False)
-    permute_alone = {
-        "gather_rows": {"GB/s": round(gather_alone[2] / gather_alone[1] / 1e6, 1),
-                        "frac_of_hbm_peak": round(gather_alone[2] / gather_alone[1] / 1e6 / HBM_PEAK_GBS, 4)},
-        "reduce_slots": {"GB/s": round(reduce_alone[2] / reduce_alone[1] / 1e6, 1),
-                         "frac_of_hbm_peak": round(reduce_alone[2] / reduce_alone[1] / 1e6 / HBM_PEAK_GBS, 4)},
-    }
-    del buf
-
-    gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_names)
-    gemm_flop = sum(kernels[k]["work_per_launch"] * kernels[k]["launches_per_step"] for k in gemm_names)
+    m = measure(cfg, args.config, device, args.steps, args.warmup, args.profile_steps, permutes_alone=True)
 
     result = {
-        "metric": "moe_mlp_fwd_bwd_tokens_per_s", "value": round(tokens_per_s, 1), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
+        "metric": "moe_mlp_fwd_bwd_tokens_per_s", "value": m["tokens_per_s"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": m["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"],
         "data": "synthetic",
         "config": {"workload": cfg["text"], "tokens": cfg["n"], "d_model": cfg["d"], "d_hidden": cfg["h"],
                    "experts": cfg["e"], "top_k": cfg["k"], "fused": cfg["fuse"],
-                   "chunks": int(os.environ["FMOE_FUSE_GRAN"]) if cfg["fuse"] else 1},
-        "roofline": roofline,
-        "gemm_all": {"tflops": round(gemm_flop / (gemm_ms * 1e-3) / 1e12, 2),
-                     "frac_of_mfma_peak": round(gemm_flop / (gemm_ms * 1e-3) / 1e12 / peak, 4),
-                     "ms_per_step": round(gemm_ms, 3)},
-        "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()}
-                    for k, v in kernels.items()},
-        "permute_alone": permute_alone,
+                   "chunks": int(os.environ["FMOE_FUSE_GRAN"]) if cfg["fuse"] else 1,
+                   "gate": "top-k over fixed seeded logits; the gate's own linear layer is not part of the step"},
+        "roofline": m["roofline"],
+        "gemm_all": m["gemm_all"],
+        "kernels": m["kernels"],
+        "permute_alone": m["permute_alone"],
         "hbm_peak_gbs": HBM_PEAK_GBS,
     }
+
+    if args.other_configs and args.config == "config4":
+        # the other workloads (parity-test configurations), 5 warm-up + 20 timed steps each
+        others = {}
+        for name in ("config1", "config2", "config3", "config5"):
+            o = measure(dict(CONFIGS[name]), name, device, 20, 5, 3, permutes_alone=False)
+            others[name] = {"workload": CONFIGS[name]["text"], "dtype": CONFIGS[name]["dtype"],
+                            "ms_per_step": o["ms_per_step"], "tokens_per_s": o["tokens_per_s"],
+                            "gemm_ms_per_step": o["gemm_all"]["ms_per_step"],
+                            "gemm_frac_of_mfma_peak": o["gemm_all"]["frac_of_mfma_peak"],
+                            "gemm_frac_of_hbm_peak": o["gemm_all"]["frac_of_hbm_peak"],
+                            "bound": o["gemm_all"]["bound"],
+                            "kernels_ms_per_step": {k: v["ms_per_step"] for k, v in o["kernels"].items()}}
+        result["other_configs"] = others
 
     if not args.no_cpu_baseline:
         from oracle import moe as omoe
