@@ -21,13 +21,14 @@ class GShardGate(NaiveGate):
     def forward(self, x):
         topk_idx, topk_val, logits = super().forward(x, return_all_scores=True)
 
+        # Balance loss.  The reference derives "top_k" as topk_idx.shape[0] // n_tokens, which is 1
+        # for the [n_tokens, 2] index tensor, so its "top-1" list is the flattened list of BOTH
+        # choices of every token (gshard_gate.py:23-31): c_e is the number of (token, choice)
+        # slots that name expert e, over the number of tokens.
         n_tokens = logits.shape[0]
-        top1_idx = topk_idx.view(-1, self.top_k)[:, 0]
-        c_e = torch.scatter_add(
-            torch.zeros(self.tot_expert, device=top1_idx.device), 0, top1_idx,
-            torch.ones_like(top1_idx, dtype=torch.float)) / n_tokens
-        m_e = torch.mean(F.softmax(logits, dim=1), dim=0)
-        self.set_loss(torch.mean(c_e * m_e) * (self.num_expert ** 2))
+        c_e = torch.bincount(topk_idx.reshape(-1), minlength=self.tot_expert).to(torch.float) / n_tokens
+        m_e = F.softmax(logits, dim=1).mean(dim=0)
+        self.set_loss((c_e * m_e).mean() * (self.num_expert ** 2))
 
         cap_rate = self.capacity[0 if self.training else 1]
         capacity = math.ceil(cap_rate * x.shape[0])

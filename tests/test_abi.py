@@ -233,3 +233,28 @@ def test_gemm_tail_plan_host_logic():
             assert 0 <= m <= tiles and 1 <= f <= 8 and (tiles - m) * f <= 256 or f == 1
             if f > 1:
                 assert per >= 16 and per * f >= slabs and per * (f - 1) < slabs and m % 256 == 0
+
+
+def test_reference_import_paths_resolve():
+    """``import fmoe`` / ``import fmoe_cuda`` and the module paths the reference's users import from."""
+    import importlib
+    import fmoe
+    import fmoe_cuda
+    import fmoe_cuda as fmoe_native_alias
+    assert fmoe_cuda is fmoe_native and fmoe_native_alias is fmoe_native
+    for name in ("expert_count", "assign_pos", "linear_forward", "linear_backward", "limit_by_capacity",
+                 "prune_gate_by_capacity", "fused_forward", "fused_backward"):
+        assert callable(getattr(fmoe_cuda, name))
+    assert fmoe.FMoE is fastermoe_amd.FMoE and fmoe.FMoETransformerMLP is fastermoe_amd.FMoETransformerMLP
+    assert fmoe.FMoELinear is fastermoe_amd.FMoELinear
+    assert fmoe.DistributedGroupedDataParallel is fastermoe_amd.DistributedGroupedDataParallel
+    from fmoe.functions import (MOECache, MOEGather, MOELinear, MOEScatter, count_by_gate, ensure_comm,  # noqa: F401
+                                prepare_forward)
+    from fmoe.fused_functions import MOEForward  # noqa: F401
+    from fmoe.gates import GShardGate, NaiveGate, NoisyGate, SwitchGate, ZeroGate  # noqa: F401
+    from fmoe.gates.utils import limit_by_capacity  # noqa: F401
+    from fmoe.layers import FMoE as LayersFMoE
+    from fmoe.transformer import FMoETransformerMLP as TransformerMLP
+    assert LayersFMoE is fastermoe_amd.FMoE and TransformerMLP is fastermoe_amd.FMoETransformerMLP
+    assert importlib.import_module("fmoe.gates.naive_gate").NaiveGate is gates.NaiveGate
+    assert importlib.import_module("fmoe.layers") is layers
