@@ -461,6 +461,33 @@ extern "C" int fmoe_linear_forward(const void *x, const void *w, const void *bia
     return grouped_linear_forward(a, expert_count_host, n_expert, 0, total, (hipStream_t)stream);
 }
 
+extern "C" int fmoe_linear_act_forward(const void *x, const void *w, const void *bias, void *pre, void *y,
+                                       const int64_t *expert_count_host, int64_t n_expert, int64_t in_feat,
+                                       int64_t out_feat, int dtype, int activation, void *stream) {
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_act_forward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(activation >= FMOE_ACT_NONE && activation <= FMOE_ACT_GELU, "fmoe_linear_act_forward: activation %d",
+                 activation);
+    int64_t total;
+    if (int rc = check_counts("fmoe_linear_act_forward", expert_count_host, n_expert, 0, 0, &total)) return rc;
+    LinearForwardArgs a{x, w, bias, y, pre, in_feat, out_feat, dtype, kEpiBiasAct, activation};
+    return grouped_linear_forward(a, expert_count_host, n_expert, 0, total, (hipStream_t)stream);
+}
+
+extern "C" int fmoe_linear_dact_backward(const void *grad_y, const void *w, const void *pre, void *grad_x,
+                                         const int64_t *expert_count_host, int64_t n_expert, int64_t in_feat,
+                                         int64_t out_feat, int dtype, int activation, void *stream) {
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_dact_backward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(activation >= FMOE_ACT_NONE && activation <= FMOE_ACT_GELU,
+                 "fmoe_linear_dact_backward: activation %d", activation);
+    int64_t total;
+    if (int rc = check_counts("fmoe_linear_dact_backward", expert_count_host, n_expert, 0, 0, &total)) return rc;
+    FMOE_REQUIRE(activation == FMOE_ACT_NONE || total == 0 || pre != nullptr, "fmoe_linear_dact_backward: pre is NULL");
+    const bool has_act = activation != FMOE_ACT_NONE;
+    LinearDgradArgs d{grad_y, w, grad_x, has_act ? pre : nullptr, in_feat, out_feat, dtype,
+                      has_act ? kEpiDAct : kEpiStore, activation};
+    return grouped_linear_dgrad(d, expert_count_host, n_expert, 0, total, (hipStream_t)stream);
+}
+
 extern "C" int fmoe_linear_backward(const void *grad_y, const void *x, const void *w, void *grad_x, void *grad_w,
                                     void *grad_b, const int64_t *expert_count_host, int64_t n_expert,
                                     int64_t in_feat, int64_t out_feat, int dtype, void *stream) {

@@ -313,6 +313,66 @@ def linear_backward(grad_output_buf, input_buf, expert_count, weight, bias=None)
     return [grad_in, grad_w, grad_b]
 
 
+def linear_act_forward(input_buf, expert_count, weight, bias, activation, keep_pre=True):
+    """``pre = X @ W_e^T + b_e`` per expert segment and ``y = act(pre)`` in one grouped GEMM
+    (the activation runs in its epilogue).  Returns ``(y, pre)``; ``pre`` is ``None`` when
+    ``keep_pre`` is false.  ``activation`` is an ``ACT_*`` code of :mod:`fastermoe_amd._lib`."""
+    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    if activation not in (_lib.ACT_NONE, _lib.ACT_RELU, _lib.ACT_GELU):
+        raise ValueError(f"unknown activation code {activation}")
+    new = lambda: torch.empty(input_buf.shape[0], out_feat, dtype=input_buf.dtype, device=input_buf.device)
+    y = new()
+    pre = new() if keep_pre else None
+    with torch.cuda.device(input_buf.device):
+        check(_lib.load().fmoe_linear_act_forward(_ptr(input_buf), _ptr(weight), _ptr(bias), _ptr(pre), _ptr(y),
+                                                  ctypes.c_void_p(cnt.data_ptr()), n_expert, in_feat, out_feat, dt,
+                                                  activation, _stream(input_buf)))
+    return y, pre
+
+
+def linear_dact_backward(grad_output_buf, expert_count, weight, pre, activation):
+    """``(grad_y @ W_e) * act'(pre)`` per expert segment: the data gradient of a linear whose input
+    was ``act(pre)``, taken with respect to ``pre``.  ``weight`` is ``[E, out_feat, in_feat]``,
+    ``pre`` ``[rows, in_feat]``."""
+    if weight.dim() != 3:
+        raise ValueError(f"weight must be [num_expert, out_feat, in_feat], got {tuple(weight.shape)}")
+    n_expert, out_feat, in_feat = weight.shape
+    dt = _rows("grad_output_buf", grad_output_buf)
+    _dev("weight", weight, grad_output_buf.dtype)
+    if grad_output_buf.shape[1] != out_feat:
+        raise ValueError(f"grad_output_buf has {grad_output_buf.shape[1]} features, weight produces {out_feat}")
+    cnt = _host_counts("expert_count", expert_count, n_expert)
+    if int(cnt.sum()) != grad_output_buf.shape[0]:
+        raise ValueError("expert_count does not sum to the number of rows")
+    if activation != _lib.ACT_NONE:
+        _dev("pre", pre, grad_output_buf.dtype)
+        if tuple(pre.shape) != (grad_output_buf.shape[0], in_feat):
+            raise ValueError(f"pre must be [{grad_output_buf.shape[0]}, {in_feat}]")
+    grad_x = torch.empty(grad_output_buf.shape[0], in_feat, dtype=grad_output_buf.dtype, device=grad_output_buf.device)
+    with torch.cuda.device(grad_output_buf.device):
+        check(_lib.load().fmoe_linear_dact_backward(_ptr(grad_output_buf), _ptr(weight),
+                                                    _ptr(pre if activation != _lib.ACT_NONE else None), _ptr(grad_x),
+                                                    ctypes.c_void_p(cnt.data_ptr()), n_expert, in_feat, out_feat, dt,
+                                                    activation, _stream(grad_output_buf)))
+    return grad_x
+
+
+def linear_weight_backward(grad_output_buf, input_buf, expert_count, weight, bias=None):
+    """The weight (and bias) half of :func:`linear_backward`: ``[grad_weight, grad_bias]``."""
+    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    _dev("grad_output_buf", grad_output_buf, input_buf.dtype)
+    if tuple(grad_output_buf.shape) != (input_buf.shape[0], out_feat):
+        raise ValueError(f"grad_output_buf must be [{input_buf.shape[0]}, {out_feat}]")
+    grad_w = torch.empty_like(weight)
+    grad_b = torch.empty(n_expert, out_feat, dtype=input_buf.dtype, device=input_buf.device) \
+        if bias is not None else None
+    with torch.cuda.device(input_buf.device):
+        check(_lib.load().fmoe_linear_backward(_ptr(grad_output_buf), _ptr(input_buf), _ptr(weight), None,
+                                               _ptr(grad_w), _ptr(grad_b), ctypes.c_void_p(cnt.data_ptr()),
+                                               n_expert, in_feat, out_feat, dt, _stream(input_buf)))
+    return [grad_w, grad_b]
+
+
 # ---- fused expert MLP (chunked, stream-overlapped pipeline) -------------------------
 
 def _mlp_params(w1, b1, w2, b2, activation):

@@ -145,6 +145,35 @@ class MOELinear(Function):
         return grad_in, None, grad_w, grad_b
 
 
+class MOEExpertMLP(Function):
+    r"""``Linear -> activation -> Linear`` of fmoe/transformer.py:22-30 over expert-sorted rows as
+    one autograd node, so that the activation runs in the first GEMM's epilogue and its
+    derivative in the epilogue of the second linear's data gradient, instead of as elementwise
+    kernels over ``[rows, d_hidden]`` of their own.  ``activation`` is an ``ACT_*`` code
+    (exact GELU, ReLU or none).  Not in the reference; same results as the three modules."""
+
+    @staticmethod
+    def forward(ctx, inp, fwd_expert_count, w1, b1, w2, b2, activation):
+        from . import _lib
+        inp = inp.contiguous()
+        keep_pre = activation == _lib.ACT_GELU  # ReLU's derivative can be read off the output
+        mid, pre = fmoe_native.linear_act_forward(inp, fwd_expert_count, w1, b1, activation, keep_pre)
+        out = fmoe_native.linear_forward(mid, fwd_expert_count, w2, b2)
+        ctx.save_for_backward(inp, fwd_expert_count, w1, b1, w2, b2, pre, mid)
+        ctx.activation = activation
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        inp, fwd_expert_count, w1, b1, w2, b2, pre, mid = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        g_pre = fmoe_native.linear_dact_backward(grad_out, fwd_expert_count, w2, pre if pre is not None else mid,
+                                                 ctx.activation)
+        gw2, gb2 = fmoe_native.linear_weight_backward(grad_out, mid, fwd_expert_count, w2, b2)
+        g_inp, gw1, gb1 = fmoe_native.linear_backward(g_pre, inp, fwd_expert_count, w1, b1)
+        return g_inp, None, gw1, gb1, gw2, gb2, None
+
+
 class MOEGather(Function):
     r"""Expert-sorted rows -> slot order, zero rows for dropped slots
     (fmoe/functions.py:278-330).  ``slot_to_row`` (optional extra) is the inverse

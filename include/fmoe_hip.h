@@ -205,6 +205,31 @@ int fmoe_linear_backward(const void *grad_y, const void *x, const void *w,
                          int64_t in_feat, int64_t out_feat, int dtype,
                          void *stream);
 
+/* The first linear of an expert MLP with its activation in the GEMM's epilogue:
+ *   pre[seg_e] = x[seg_e] . w[e]^T + bias[e]   (stored when pre != NULL)
+ *   y[seg_e]   = act(pre[seg_e])
+ * Replaces FMoELinear followed by the activation module as two kernels,
+ * fmoe/transformer.py:22-30 (_Expert.forward: htoh4, activation). */
+int fmoe_linear_act_forward(const void *x, const void *w, const void *bias,
+                            void *pre, void *y,
+                            const int64_t *expert_count_host, int64_t n_expert,
+                            int64_t in_feat, int64_t out_feat, int dtype,
+                            int activation, void *stream);
+
+/* Data gradient of the second linear with the activation's derivative in the
+ * epilogue: grad_x[seg_e] = (grad_y[seg_e] . w[e]) * act'(pre[seg_e]), i.e. the
+ * gradient with respect to the first linear's pre-activation.  w is
+ * [E, out_feat, in_feat], pre and grad_x are [rows, in_feat].  For ReLU the
+ * post-activation may be passed as pre (same sign pattern).  Replaces the
+ * data-grad half of fmoe_cuda_linear_backward_impl,
+ * cuda/parallel_linear.cuh:122-132, followed by torch's activation backward
+ * (autograd of fmoe/transformer.py:22-30). */
+int fmoe_linear_dact_backward(const void *grad_y, const void *w, const void *pre,
+                              void *grad_x, const int64_t *expert_count_host,
+                              int64_t n_expert, int64_t in_feat,
+                              int64_t out_feat, int dtype, int activation,
+                              void *stream);
+
 /* How a forward / data-grad launch of `total_tiles` output tiles (256 x 256, or
  * 128 x 256 for small launches) with `contraction_slabs` slabs of 128
  * contraction bytes is spread over `compute_units` (0: the current device's):

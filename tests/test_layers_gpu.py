@@ -138,6 +138,44 @@ def test_transformer_mlp_configs(fuse, dtype, n, d, h, e, k, act, device):
     _compare(moe, x, act, k, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("act", ["gelu", "relu", "none", "tanh"])
+def test_expert_epilogue_node_matches_the_three_modules(dtype, act, device, monkeypatch):
+    """_Expert runs Linear -> activation -> Linear as one autograd node with the activation in the
+    GEMM epilogues when the activation is the exact GELU, ReLU or none; FMOE_EXPERT_EPILOGUE=0 (and
+    any other activation, here tanh) runs the reference's three modules (fmoe/transformer.py:22-30).
+    Both against each other and, for GELU / ReLU, against the float64 oracle."""
+    torch.manual_seed(31)
+    n, d, h, e, k = 333, 96, 160, 5, 2
+    module = {"gelu": nn.GELU(), "relu": nn.ReLU(), "none": nn.Identity(), "tanh": nn.Tanh()}[act]
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=module)
+    with torch.no_grad():
+        moe.experts.htoh4.weight.mul_((d * h) ** 0.5 * d ** -0.5)
+        moe.experts.h4toh.weight.mul_((d * h) ** 0.5 * h ** -0.5)
+        moe.experts.htoh4.bias.normal_(0, 0.3)
+        moe.experts.h4toh.bias.normal_(0, 0.3)
+    moe = moe.to(dtype).to(device)
+    assert (moe.experts._epilogue_activation() is None) == (act == "tanh")
+    x = torch.randn(n, d).to(dtype).to(device)
+    idx = torch.randint(-1, e - 1, (n, k), device=device)     # drops, and expert e-1 without rows
+    score = torch.rand(n, k, device=device).to(dtype)
+    moe.gate.forward = lambda inp: (idx, score)
+    results = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("FMOE_EXPERT_EPILOGUE", flag)
+        moe.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        out.float().mean().backward()
+        results.append([out, xi.grad] + [p.grad.clone() for p in moe.experts.parameters()])
+    tol = TOL[dtype]
+    for a, b in zip(*results):
+        assert rel_err(a, b) <= (2 * tol if dtype == torch.bfloat16 else 10 * tol)
+    if act in ("gelu", "relu"):
+        monkeypatch.setenv("FMOE_EXPERT_EPILOGUE", "1")
+        _compare(moe, x, act, k, dtype)
+
+
 @pytest.mark.parametrize("fuse", [False, True])
 @pytest.mark.parametrize("n,d,h,e,k,routing", [
     (1024, 2048, 8192, 64, 1, "zipf"),     # the skewed Switch-style layer at full width: Zipf(1.2) top-1, empty experts
@@ -386,7 +424,7 @@ def test_gshard_gate(cap, n, e, device):
     limit = math.ceil(cap * n)
     counts = torch.bincount(idx[idx >= 0].view(-1), minlength=e)
     assert int(counts.max()) <= limit
-    logits = gate.gate(x)
+    logits = gate.gate(x).detach()
     kept = idx >= 0
     assert torch.equal(torch.gather(logits, 1, idx.clamp(min=0))[kept], val[kept])
     # the balance loss of fmoe/gates/gshard_gate.py:23-34 in closed form: both choices of every token counted
@@ -394,7 +432,7 @@ def test_gshard_gate(cap, n, e, device):
     c_e = torch.bincount(top_idx.reshape(-1), minlength=e).double() / n
     m_e = torch.softmax(logits.double(), dim=1).mean(0)
     want_loss = float((c_e * m_e).sum() / e * e * e)
-    assert abs(float(gate.get_loss()) - want_loss) <= 1e-5 * want_loss
+    assert abs(float(gate.get_loss().detach()) - want_loss) <= 1e-5 * want_loss
     assert abs(float(c_e.sum()) - 2.0) < 1e-9
     # first-come-first-kept: what survives the capacity step is the oracle's pruning
     top_val, top_idx = torch.topk(logits, 2, dim=-1, sorted=False)
