@@ -47,6 +47,7 @@ def build_layer(cfg, device):
     import torch
     import fastermoe_amd as fmoe
     from fastermoe_amd.gates.base_gate import BaseGate
+    from fastermoe_amd.functions import gate_topk
     from fastermoe_amd.gates.utils import limit_by_capacity
 
     dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
@@ -71,8 +72,8 @@ def build_layer(cfg, device):
             self.top_k = top_k
 
         def forward(self, inp):
-            val, idx = torch.topk(logits, k=self.top_k, dim=-1)
-            score = torch.softmax(val, dim=-1).to(inp.dtype)
+            idx, score = gate_topk(logits, self.top_k, score_mode=1)
+            score = score.to(inp.dtype)
             if "cap" in cfg:
                 _, _, idx = limit_by_capacity(idx, self.num_expert, 1, cfg["cap"])
             return idx, score

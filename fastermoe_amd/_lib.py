@@ -32,6 +32,8 @@ SIGNATURES = {
     "fmoe_assign_pos": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
     "fmoe_route": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp]),
     "fmoe_route_static": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "fmoe_gate_topk_route": (_int, [_vp, _i64, _i64, _i64, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "fmoe_gate_topk_backward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     "fmoe_limit_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "fmoe_prune_gate_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp]),
     "fmoe_gather_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),

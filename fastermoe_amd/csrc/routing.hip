@@ -48,48 +48,82 @@ __device__ __forceinline__ uint64_t match_mask(int key, bool valid, int nbits) {
     return valid ? peers : 0ull;
 }
 
+// Orders this wave's LDS accesses: the lanes of a wave run in lock-step and the LDS serves a
+// wave's instructions in order, so a wave-private table needs no workgroup barrier -- only
+// the compiler must keep the accesses in program order.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// Adds this wave's 64 keys to its private table without atomics: of the lanes that hold the
+// same key, the lowest one adds their number.
+__device__ __forceinline__ void wave_bins_add(int32_t *mine, int key, bool valid, uint64_t peers) {
+    if (valid && (peers & lanes_below()) == 0) mine[key] += __popcll(peers);
+    wave_lds_sync();
+}
+
 // ---------------------------------------------------------------- count ----
 
-// LDS histogram per workgroup, one global integer add per non-empty bin.
+// Wave-private LDS histograms filled without atomics, then one global integer add per
+// workgroup and non-empty bin (the entry point ADDS to the caller's counts, as the
+// reference kernel does; integer adds commute, so the result does not depend on scheduling).
 __global__ __launch_bounds__(kBlock) void expert_count_kernel(
     const int64_t *__restrict__ gate, int32_t *__restrict__ count,
-    int64_t n_slots, int n_expert) {
-    extern __shared__ int32_t bins[];
-    for (int e = threadIdx.x; e < n_expert; e += kBlock) bins[e] = 0;
+    int64_t n_slots, int n_expert, int nbits) {
+    extern __shared__ int32_t bins[];  // [kWavesPerBlock][n_expert]
+    int32_t *mine = bins + (threadIdx.x / kWave) * n_expert;
+    for (int e = threadIdx.x; e < kWavesPerBlock * n_expert; e += kBlock) bins[e] = 0;
     __syncthreads();
     const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n_slots; i += stride) {
-        const int64_t g = gate[i];
-        if (g >= 0 && g < n_expert) atomicAdd(&bins[(int)g], 1);
+    const int64_t rounds = (n_slots + stride - 1) / stride;  // the same for every lane: ballots need whole waves
+    for (int64_t r = 0; r < rounds; ++r) {
+        const int64_t i = r * stride + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+        int64_t g = -1;
+        if (i < n_slots) g = gate[i];
+        const bool valid = g >= 0 && g < n_expert;
+        const int key = valid ? (int)g : 0;
+        wave_bins_add(mine, key, valid, match_mask(key, valid, nbits));
     }
     __syncthreads();
     for (int e = threadIdx.x; e < n_expert; e += kBlock) {
-        const int32_t c = bins[e];
+        int32_t c = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) c += bins[w * n_expert + e];
         if (c) atomicAdd(&count[e], c);
     }
 }
 
 // ----------------------------------------------------------------- hist ----
 
-// block_hist[b][e] = #slots of expert e in workgroup b's slot range.
+// block_hist[b][e] = #slots of expert e in workgroup b's slot range; wave-private tables
+// filled without atomics, added up at the end.
 __global__ __launch_bounds__(kBlock) void block_hist_kernel(
     const int64_t *__restrict__ gate, int32_t *__restrict__ block_hist,
-    int64_t n_slots, int n_expert) {
-    extern __shared__ int32_t bins[];
-    for (int e = threadIdx.x; e < n_expert; e += kBlock) bins[e] = 0;
+    int64_t n_slots, int n_expert, int nbits) {
+    extern __shared__ int32_t bins[];  // [kWavesPerBlock][n_expert]
+    const int wave = threadIdx.x / kWave;
+    int32_t *mine = bins + wave * n_expert;
+    for (int e = threadIdx.x; e < kWavesPerBlock * n_expert; e += kBlock) bins[e] = 0;
     __syncthreads();
-    const int64_t base = (int64_t)blockIdx.x * kSlotsPerBlock;
+    const int64_t wave_base = (int64_t)blockIdx.x * kSlotsPerBlock + (int64_t)wave * kSlotsPerWave;
 #pragma unroll
-    for (int s = 0; s < kSlotsPerBlock / kBlock; ++s) {
-        const int64_t i = base + s * kBlock + threadIdx.x;
-        if (i < n_slots) {
-            const int64_t g = gate[i];
-            if (g >= 0 && g < n_expert) atomicAdd(&bins[(int)g], 1);
-        }
+    for (int s = 0; s < kStepsPerWave; ++s) {
+        const int64_t i = wave_base + s * kWave + lane_id();
+        int64_t g = -1;
+        if (i < n_slots) g = gate[i];
+        const bool valid = g >= 0 && g < n_expert;
+        const int key = valid ? (int)g : 0;
+        wave_bins_add(mine, key, valid, match_mask(key, valid, nbits));
     }
     __syncthreads();
     int32_t *dst = block_hist + (int64_t)blockIdx.x * n_expert;
-    for (int e = threadIdx.x; e < n_expert; e += kBlock) dst[e] = bins[e];
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) {
+        int32_t c = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) c += bins[w * n_expert + e];
+        dst[e] = c;
+    }
 }
 
 // ----------------------------------------------------------------- scan ----
@@ -181,13 +215,15 @@ __global__ __launch_bounds__(kBlock) void rank_apply_kernel(
 
     const int64_t wave_base = (int64_t)blockIdx.x * kSlotsPerBlock + (int64_t)wave * kSlotsPerWave;
     int keys[kStepsPerWave];
+    uint64_t peers[kStepsPerWave];
 #pragma unroll
     for (int s = 0; s < kStepsPerWave; ++s) {
         const int64_t i = wave_base + s * kWave + lane_id();
         int64_t g = -1;
         if (i < n_slots) g = gate[i];
         keys[s] = (g >= 0 && g < n_expert) ? (int)g : -1;
-        if (keys[s] >= 0) atomicAdd(&mine[keys[s]], 1);
+        peers[s] = match_mask(keys[s], keys[s] >= 0, nbits);
+        wave_bins_add(mine, keys[s], keys[s] >= 0, peers[s]);
     }
     __syncthreads();
     // per-wave histogram -> starting rank of this wave for every expert
@@ -203,17 +239,16 @@ __global__ __launch_bounds__(kBlock) void rank_apply_kernel(
     }
     __syncthreads();
 
+    // from here on a wave only touches its own table: wave-level ordering is enough
 #pragma unroll
     for (int s = 0; s < kStepsPerWave; ++s) {
         const int64_t i = wave_base + s * kWave + lane_id();
         const int key = keys[s];
         const bool valid = key >= 0;
-        const uint64_t peers = match_mask(key, valid, nbits);
         int32_t rank = 0;
-        if (valid) rank = mine[key] + __popcll(peers & lanes_below());
-        __syncthreads();  // every lane has read its counter before leaders bump it
-        if (valid && (peers & lanes_below()) == 0) mine[key] += __popcll(peers);
-        __syncthreads();
+        if (valid) rank = mine[key] + __popcll(peers[s] & lanes_below());
+        wave_lds_sync();  // every lane has read its counter before the leaders bump it
+        wave_bins_add(mine, key, valid, peers[s]);
         if (MODE == kApplyAssign) {
             if (valid) {
                 const int64_t row = (int64_t)limit_old[key] - 1 - rank;
@@ -226,6 +261,110 @@ __global__ __launch_bounds__(kBlock) void rank_apply_kernel(
             if (i < n_slots) out[i] = (valid && rank < limit_old[key]) ? (int64_t)key : -1;
         }
     }
+}
+
+// ----------------------------------------------------------------- gate ----
+
+// Top-k of the gate logits, the scores of the selected experts and the per-workgroup expert
+// histogram that the routing scan starts from, in one pass over the logits.
+//
+// A workgroup owns kSlotsPerBlock consecutive (token, choice) slots -- the same slots as
+// workgroup b of rank_apply_kernel -- a wave kSlotsPerWave of them.  A token is worked on by a
+// group of G lanes (G = the power of two at or above n_expert, at most 64), lane g of the group
+// holding logits g, g + G, ...: round j finds the largest remaining logit of the group by
+// xor-shuffles (ties go to the lower expert index), lane j keeps it, and the owner strikes it
+// out.  Lanes 0 .. top_k-1 of a group then hold the token's choices in descending order of the
+// logit; they write index and score, and the wave adds their keys to its private table.
+// score_mode 0: the selected logit itself; 1: softmax over the top_k selected logits.
+template <typename T, int VPL>
+__global__ __launch_bounds__(kBlock) void gate_topk_hist_kernel(
+    const T *__restrict__ logits, int64_t n_tokens, int n_expert, int top_k, int group, int score_mode,
+    int64_t *__restrict__ topk_idx, T *__restrict__ topk_score, int32_t *__restrict__ block_hist, int nbits) {
+    extern __shared__ int32_t bins[];  // [kWavesPerBlock][n_expert]
+    const int wave = threadIdx.x / kWave;
+    int32_t *mine = bins + wave * n_expert;
+    for (int e = threadIdx.x; e < kWavesPerBlock * n_expert; e += kBlock) bins[e] = 0;
+    __syncthreads();
+
+    const int lane = lane_id();
+    const int g = lane & (group - 1), sub = lane / group;     // lane in its group, group in the wave
+    const int tokens_per_step = kWave / group;
+    const int64_t wave_token0 = ((int64_t)blockIdx.x * kSlotsPerBlock + (int64_t)wave * kSlotsPerWave) / top_k;
+    const int steps = kSlotsPerWave / top_k / tokens_per_step;
+    const float kLowest = -__builtin_inff();
+
+    for (int s = 0; s < steps; ++s) {
+        const int64_t token = wave_token0 + (int64_t)s * tokens_per_step + sub;
+        const bool live = token < n_tokens;
+        float v[VPL];
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int e = g + i * group;
+            v[i] = (live && e < n_expert) ? (float)logits[token * n_expert + e] : kLowest;
+        }
+        float my_v = kLowest, v_max = 0.f;
+        int my_e = -1;
+        for (int j = 0; j < top_k; ++j) {
+            float best = v[0];
+            int best_e = g;
+#pragma unroll
+            for (int i = 1; i < VPL; ++i)
+                if (v[i] > best) { best = v[i]; best_e = g + i * group; }
+            for (int m = 1; m < group; m <<= 1) {
+                const float ov = __shfl_xor(best, m, kWave);
+                const int oe = __shfl_xor(best_e, m, kWave);
+                if (ov > best || (ov == best && oe < best_e)) { best = ov; best_e = oe; }
+            }
+            if (j == 0) v_max = best;
+            if (g == j) { my_v = best; my_e = best_e; }
+#pragma unroll
+            for (int i = 0; i < VPL; ++i)
+                if (g + i * group == best_e) v[i] = kLowest;
+        }
+        const bool chosen = live && g < top_k && my_e >= 0 && my_e < n_expert;
+        float score = my_v;
+        if (score_mode == 1) {
+            float ex = chosen ? __expf(my_v - v_max) : 0.f, sum = ex;
+            for (int m = 1; m < group; m <<= 1) sum += __shfl_xor(sum, m, kWave);
+            score = ex / sum;
+        }
+        if (live && g < top_k) {
+            topk_idx[token * top_k + g] = chosen ? (int64_t)my_e : -1;
+            topk_score[token * top_k + g] = (T)(chosen ? score : 0.f);
+        }
+        wave_bins_add(mine, chosen ? my_e : 0, chosen, match_mask(chosen ? my_e : 0, chosen, nbits));
+    }
+    __syncthreads();
+    int32_t *dst = block_hist + (int64_t)blockIdx.x * n_expert;
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) {
+        int32_t c = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) c += bins[w * n_expert + e];
+        dst[e] = c;
+    }
+}
+
+// Gradient of the scores with respect to the logits: zero except at the selected experts.
+// score_mode 0: grad_logits[t, idx[t,j]] = grad_score[t,j];
+// score_mode 1: grad_logits[t, idx[t,j]] = score[t,j] * (grad_score[t,j] - sum_i grad_score[t,i] score[t,i]).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gate_topk_backward_kernel(
+    const T *__restrict__ grad_score, const T *__restrict__ score, const int64_t *__restrict__ topk_idx,
+    T *__restrict__ grad_logits, int64_t n_tokens, int n_expert, int top_k, int score_mode) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_tokens * n_expert) return;
+    const int64_t t = i / n_expert;
+    const int e = (int)(i - t * n_expert);
+    float dot = 0.f;
+    if (score_mode == 1)
+        for (int j = 0; j < top_k; ++j) dot += (float)grad_score[t * top_k + j] * (float)score[t * top_k + j];
+    float gval = 0.f;
+    for (int j = 0; j < top_k; ++j)
+        if (topk_idx[t * top_k + j] == e) {
+            const float gs = (float)grad_score[t * top_k + j];
+            gval = score_mode == 1 ? (float)score[t * top_k + j] * (gs - dot) : gs;
+        }
+    grad_logits[i] = (T)gval;
 }
 
 // ------------------------------------------------------------- capacity ----
@@ -259,6 +398,13 @@ int ilog2_ceil(int64_t n) {
     int b = 0;
     while ((1ll << b) < n) ++b;
     return b < 1 ? 1 : b;
+}
+
+// Dynamic LDS beyond 64 KiB (more than 4096 experts) has to be allowed per kernel.
+int allow_lds(const void *kernel, size_t bytes) {
+    if (bytes <= 64 * 1024) return FMOE_OK;
+    FMOE_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    return FMOE_OK;
 }
 
 struct RouteScratch {
@@ -310,8 +456,10 @@ extern "C" int fmoe_expert_count(const int64_t *gate_idx, int32_t *expert_count,
     FMOE_REQUIRE(gate_idx && expert_count, "fmoe_expert_count: NULL pointer");
     const int64_t blocks = ceil_div(n_slots, (int64_t)kBlock * 8);
     const int grid = (int)(blocks < 1024 ? blocks : 1024);
-    expert_count_kernel<<<grid, kBlock, n_expert * sizeof(int32_t), (hipStream_t)stream>>>(
-        gate_idx, expert_count, n_slots, (int)n_expert);
+    const size_t lds = kWavesPerBlock * n_expert * sizeof(int32_t);
+    if (int rc = allow_lds((const void *)expert_count_kernel, lds)) return rc;
+    expert_count_kernel<<<grid, kBlock, lds, (hipStream_t)stream>>>(
+        gate_idx, expert_count, n_slots, (int)n_expert, ilog2_ceil(n_expert));
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
 }
@@ -331,10 +479,12 @@ extern "C" int fmoe_assign_pos(int32_t *cum_count, const int64_t *gate, int64_t 
     if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
     hipStream_t st = (hipStream_t)stream;
     const int E = (int)n_expert;
-    block_hist_kernel<<<s.n_blocks, kBlock, E * sizeof(int32_t), st>>>(gate, s.block_hist, n_slots, E);
+    if (int rc = allow_lds((const void *)block_hist_kernel, kWavesPerBlock * E * sizeof(int32_t))) return rc;
+    block_hist_kernel<<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(gate, s.block_hist, n_slots, E, ilog2_ceil(n_expert));
     FMOE_LAUNCH_CHECK();
     block_scan_kernel<<<(int)ceil_div(E, kBlock), kBlock, 0, st>>>(s.block_hist, s.n_blocks, E, cum_count, s.limit_old);
     FMOE_LAUNCH_CHECK();
+    if (int rc = allow_lds((const void *)rank_apply_kernel<kApplyAssign>, kWavesPerBlock * E * sizeof(int32_t))) return rc;
     rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
         gate, s.block_hist, s.limit_old, pos, nullptr, n_slots, n_pos, E, ilog2_ceil(n_expert));
     FMOE_LAUNCH_CHECK();
@@ -348,10 +498,12 @@ namespace {
 int route_launch(const int64_t *gate, int64_t n_slots, int64_t n_expert, int64_t *expert_count, int64_t *pos,
                  int64_t *slot_to_row, const RouteScratch &s, hipStream_t st) {
     const int E = (int)n_expert;
-    block_hist_kernel<<<s.n_blocks, kBlock, E * sizeof(int32_t), st>>>(gate, s.block_hist, n_slots, E);
+    if (int rc = allow_lds((const void *)block_hist_kernel, kWavesPerBlock * E * sizeof(int32_t))) return rc;
+    block_hist_kernel<<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(gate, s.block_hist, n_slots, E, ilog2_ceil(n_expert));
     FMOE_LAUNCH_CHECK();
     route_scan_kernel<<<1, kRouteScanBlock, 0, st>>>(s.block_hist, s.n_blocks, E, expert_count, s.cum);
     FMOE_LAUNCH_CHECK();
+    if (int rc = allow_lds((const void *)rank_apply_kernel<kApplyAssign>, kWavesPerBlock * E * sizeof(int32_t))) return rc;
     rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
         gate, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert));
     FMOE_LAUNCH_CHECK();
@@ -449,12 +601,105 @@ extern "C" int fmoe_prune_gate_by_capacity(const int64_t *gate_idx, int64_t *new
     if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
     hipStream_t st = (hipStream_t)stream;
     const int E = (int)n_expert;
-    block_hist_kernel<<<s.n_blocks, kBlock, E * sizeof(int32_t), st>>>(gate_idx, s.block_hist, n_slots, E);
+    if (int rc = allow_lds((const void *)block_hist_kernel, kWavesPerBlock * E * sizeof(int32_t))) return rc;
+    block_hist_kernel<<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(gate_idx, s.block_hist, n_slots, E, ilog2_ceil(n_expert));
     FMOE_LAUNCH_CHECK();
     block_scan_kernel<<<(int)ceil_div(E, kBlock), kBlock, 0, st>>>(s.block_hist, s.n_blocks, E, ec, s.limit_old);
     FMOE_LAUNCH_CHECK();
+    if (int rc = allow_lds((const void *)rank_apply_kernel<kApplyPrune>, kWavesPerBlock * E * sizeof(int32_t))) return rc;
     rank_apply_kernel<kApplyPrune><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
         gate_idx, s.block_hist, s.limit_old, new_gate_idx, nullptr, n_slots, n_slots, E, ilog2_ceil(n_expert));
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+
+namespace fmoe {
+namespace {
+
+template <typename T>
+int launch_gate_topk(const void *logits, int64_t n_tokens, int E, int top_k, int score_mode, int64_t *topk_idx,
+                     void *topk_score, int32_t *block_hist, int n_blocks, hipStream_t st) {
+    int group = 1;
+    while (group < E && group < kWave) group <<= 1;
+    const int vpl = (int)ceil_div(E, group);
+    const size_t lds = kWavesPerBlock * E * sizeof(int32_t);
+    const int nbits = ilog2_ceil(E);
+#define FMOE_GATE_LAUNCH(V)                                                                                       \
+    do {                                                                                                          \
+        if (int rc = allow_lds((const void *)gate_topk_hist_kernel<T, V>, lds)) return rc;                        \
+        gate_topk_hist_kernel<T, V><<<n_blocks, kBlock, lds, st>>>((const T *)logits, n_tokens, E, top_k, group,  \
+                                                                   score_mode, topk_idx, (T *)topk_score,         \
+                                                                   block_hist, nbits);                            \
+    } while (0)
+    if (vpl <= 1) FMOE_GATE_LAUNCH(1);
+    else if (vpl <= 2) FMOE_GATE_LAUNCH(2);
+    else if (vpl <= 4) FMOE_GATE_LAUNCH(4);
+    else if (vpl <= 8) FMOE_GATE_LAUNCH(8);
+    else FMOE_GATE_LAUNCH(16);
+#undef FMOE_GATE_LAUNCH
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+}  // namespace
+}  // namespace fmoe
+
+extern "C" int fmoe_gate_topk_route(const void *logits, int64_t n_tokens, int64_t n_expert, int64_t top_k, int dtype,
+                                    int score_mode, int64_t *topk_idx, void *topk_score, int64_t *expert_count,
+                                    int64_t *pos, int64_t *slot_to_row, void *workspace, int64_t workspace_bytes,
+                                    void *stream) {
+    FMOE_REQUIRE(n_tokens >= 0 && top_k >= 1, "fmoe_gate_topk_route: n_tokens=%lld top_k=%lld", (long long)n_tokens,
+                 (long long)top_k);
+    FMOE_REQUIRE(dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16, "fmoe_gate_topk_route: dtype %d", dtype);
+    FMOE_REQUIRE(score_mode == 0 || score_mode == 1, "fmoe_gate_topk_route: score_mode %d", score_mode);
+    if (n_expert < 1 || n_expert > 16 * kWave)
+        return fail(FMOE_ELIMIT, "fmoe_gate_topk_route: %lld experts (1..%d)", (long long)n_expert, 16 * kWave);
+    if (top_k > n_expert || top_k > kWave || (top_k & (top_k - 1)) != 0)
+        return fail(FMOE_ELIMIT, "fmoe_gate_topk_route: top_k=%lld must be a power of two, at most 64 and at most n_expert",
+                    (long long)top_k);
+    const int64_t n_slots = n_tokens * top_k;
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    FMOE_REQUIRE(expert_count, "fmoe_gate_topk_route: NULL expert_count");
+    hipStream_t st = (hipStream_t)stream;
+    if (n_slots == 0) return route_empty(n_expert, expert_count, st);
+    FMOE_REQUIRE(logits && topk_idx && topk_score && pos, "fmoe_gate_topk_route: NULL pointer");
+    RouteScratch s;
+    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+    const int E = (int)n_expert;
+    int rc = FMOE_OK;
+    switch (dtype) {
+        case FMOE_F32: rc = launch_gate_topk<float>(logits, n_tokens, E, (int)top_k, score_mode, topk_idx, topk_score, s.block_hist, s.n_blocks, st); break;
+        case FMOE_BF16: rc = launch_gate_topk<__bf16>(logits, n_tokens, E, (int)top_k, score_mode, topk_idx, topk_score, s.block_hist, s.n_blocks, st); break;
+        default: rc = launch_gate_topk<_Float16>(logits, n_tokens, E, (int)top_k, score_mode, topk_idx, topk_score, s.block_hist, s.n_blocks, st); break;
+    }
+    if (rc) return rc;
+    route_scan_kernel<<<1, kRouteScanBlock, 0, st>>>(s.block_hist, s.n_blocks, E, expert_count, s.cum);
+    FMOE_LAUNCH_CHECK();
+    if (int rc2 = allow_lds((const void *)rank_apply_kernel<kApplyAssign>, kWavesPerBlock * E * sizeof(int32_t))) return rc2;
+    rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
+        topk_idx, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert));
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_gate_topk_backward(const void *grad_score, const void *score, const int64_t *topk_idx,
+                                       void *grad_logits, int64_t n_tokens, int64_t n_expert, int64_t top_k,
+                                       int dtype, int score_mode, void *stream) {
+    FMOE_REQUIRE(n_tokens >= 0 && n_expert >= 1 && top_k >= 1, "fmoe_gate_topk_backward: bad sizes");
+    FMOE_REQUIRE(dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16, "fmoe_gate_topk_backward: dtype %d", dtype);
+    FMOE_REQUIRE(score_mode == 0 || score_mode == 1, "fmoe_gate_topk_backward: score_mode %d", score_mode);
+    const int64_t n = n_tokens * n_expert;
+    if (n == 0) return FMOE_OK;
+    if (n > (int64_t)INT32_MAX * kBlock) return fail(FMOE_ELIMIT, "fmoe_gate_topk_backward: %lld logits", (long long)n);
+    FMOE_REQUIRE(grad_score && topk_idx && grad_logits && (score_mode == 0 || score), "fmoe_gate_topk_backward: NULL pointer");
+    const unsigned grid = (unsigned)ceil_div(n, kBlock);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case FMOE_F32: gate_topk_backward_kernel<float><<<grid, kBlock, 0, st>>>((const float *)grad_score, (const float *)score, topk_idx, (float *)grad_logits, n_tokens, (int)n_expert, (int)top_k, score_mode); break;
+        case FMOE_BF16: gate_topk_backward_kernel<__bf16><<<grid, kBlock, 0, st>>>((const __bf16 *)grad_score, (const __bf16 *)score, topk_idx, (__bf16 *)grad_logits, n_tokens, (int)n_expert, (int)top_k, score_mode); break;
+        default: gate_topk_backward_kernel<_Float16><<<grid, kBlock, 0, st>>>((const _Float16 *)grad_score, (const _Float16 *)score, topk_idx, (_Float16 *)grad_logits, n_tokens, (int)n_expert, (int)top_k, score_mode); break;
+    }
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
 }

@@ -106,6 +106,54 @@ def route(gate, n_expert):
     return cnt, pos, s2r
 
 
+def gate_topk_supported(n_expert, top_k, dtype):
+    """Whether :func:`gate_topk_route` takes this gate shape (else: torch.topk and :func:`route`)."""
+    return (1 <= top_k <= min(n_expert, 64) and top_k & (top_k - 1) == 0 and n_expert <= 1024
+            and dtype in (torch.float32, torch.bfloat16, torch.float16))
+
+
+def gate_topk_route(logits, top_k, score_mode=0):
+    """Top-k of ``logits [N, E]`` with the routing bookkeeping in the same launches.  Returns
+    ``(topk_idx int64 [N,k], topk_score [N,k], expert_count int64 [E], pos_buf int64 [N*k],
+    slot_to_row int64 [N*k])``; ``score_mode`` 0 returns the selected logits as scores, 1 their
+    softmax over the k selected."""
+    _dev("logits", logits)
+    if logits.dim() != 2:
+        raise ValueError(f"logits must be [n_tokens, n_expert], got {tuple(logits.shape)}")
+    n, e = logits.shape
+    if not gate_topk_supported(e, top_k, logits.dtype):
+        raise ValueError(f"gate_topk_route does not take n_expert={e}, top_k={top_k}, dtype={logits.dtype}")
+    dt = _float_dtype("logits", logits)
+    lib = _lib.load()
+    dev = logits.device
+    with torch.cuda.device(dev):
+        idx = torch.empty(n, top_k, dtype=torch.int64, device=dev)
+        score = torch.empty(n, top_k, dtype=logits.dtype, device=dev)
+        cnt = torch.empty(e, dtype=torch.int64, device=dev)
+        pos = torch.empty(n * top_k, dtype=torch.int64, device=dev)
+        s2r = torch.empty(n * top_k, dtype=torch.int64, device=dev)
+        ws = _workspace(lib.fmoe_routing_workspace_bytes(n * top_k, e), dev)
+        check(lib.fmoe_gate_topk_route(_ptr(logits), n, e, top_k, dt, score_mode, _ptr(idx), _ptr(score), _ptr(cnt),
+                                       _ptr(pos), _ptr(s2r), _ptr(ws), ws.numel(), _stream(logits)))
+    return idx, score, cnt, pos, s2r
+
+
+def gate_topk_backward(grad_score, score, topk_idx, n_expert, score_mode=0):
+    """Gradient of the top-k scores with respect to the logits, ``[N, E]``."""
+    _dev("grad_score", grad_score)
+    _dev("topk_idx", topk_idx, torch.int64)
+    n, k = topk_idx.shape
+    dt = _float_dtype("grad_score", grad_score)
+    if score_mode == 1:
+        _dev("score", score, grad_score.dtype)
+    grad_logits = torch.empty(n, n_expert, dtype=grad_score.dtype, device=grad_score.device)
+    with torch.cuda.device(grad_score.device):
+        check(_lib.load().fmoe_gate_topk_backward(_ptr(grad_score), _ptr(score if score_mode == 1 else None),
+                                                  _ptr(topk_idx), _ptr(grad_logits), n, n_expert, k, dt, score_mode,
+                                                  _stream(grad_score)))
+    return grad_logits
+
+
 def limit_by_capacity(expert_count, capacity, n_expert, n_worker):
     """fmoe_cuda.limit_by_capacity, cuda/balancing.cu:7-20."""
     _dev("expert_count", expert_count, torch.int64)

@@ -23,13 +23,54 @@ def ensure_comm(t, comm):
     return None
 
 
+class GateTopK(Function):
+    r"""``torch.topk`` of the gate logits (and, with ``score_mode`` 1, the softmax over the selected
+    logits) of fmoe/gates/naive_gate.py:26-42 with the routing of ``count_by_gate`` computed in
+    the same launches.  Returns ``(topk_idx [N,k], topk_score [N,k])``; the routing result rides
+    on ``topk_idx`` (``_fmoe_route``) and is picked up by :func:`_route` when the layer is handed
+    this very tensor, unmodified."""
+
+    @staticmethod
+    def forward(ctx, logits, top_k, score_mode):
+        logits = logits.contiguous()
+        idx, score, cnt, pos_buf, s2r = fmoe_native.gate_topk_route(logits, top_k, score_mode)
+        ctx.save_for_backward(idx, score)
+        ctx.moe_args = logits.shape[1], score_mode
+        ctx.mark_non_differentiable(idx)
+        idx._fmoe_route = (idx._version, logits.shape[1], cnt, pos_buf, s2r)
+        return idx, score
+
+    @staticmethod
+    def backward(ctx, _grad_idx, grad_score):
+        idx, score = ctx.saved_tensors
+        n_expert, score_mode = ctx.moe_args
+        return fmoe_native.gate_topk_backward(grad_score.contiguous(), score, idx, n_expert, score_mode), None, None
+
+
+def gate_topk(logits, top_k, score_mode=0):
+    r"""Top-k indices and scores of ``logits [N, E]``: the HIP gate kernel when it takes the shape
+    (CUDA tensor, 16/32-bit floats, ``top_k`` a power of two, at most 1024 experts), ``torch.topk``
+    otherwise.  ``score_mode`` 0: the selected logits; 1: their softmax over the ``top_k``."""
+    if logits.is_cuda and logits.dim() == 2 and fmoe_native.gate_topk_supported(logits.shape[1], top_k, logits.dtype):
+        idx, score = GateTopK.apply(logits, top_k, score_mode)
+        # autograd hands back a new Python object for the index tensor: carry the routing over
+        return idx, score
+    val, idx = torch.topk(logits, k=top_k, dim=-1, largest=True, sorted=False)
+    return idx, (torch.softmax(val, dim=-1) if score_mode == 1 else val)
+
+
 def _route(gate, num_expert, world_size):
     """(pos, counts, slot_to_row): one fused routing call and ONE device-to-host
     read (the counts), instead of the histogram / cumsum / ``.item()`` /
-    placement sequence of fmoe/functions.py:19-42."""
+    placement sequence of fmoe/functions.py:19-42.  An index tensor that comes
+    straight from :class:`GateTopK` carries its routing with it."""
     _single_worker(world_size, "count_by_gate")
     with torch.no_grad():
-        counts, pos_buf, slot_to_row = fmoe_native.route(gate.contiguous(), num_expert)
+        cached = getattr(gate, "_fmoe_route", None)
+        if cached is not None and cached[0] == gate._version and cached[1] == num_expert:
+            counts, pos_buf, slot_to_row = cached[2:]
+        else:
+            counts, pos_buf, slot_to_row = fmoe_native.route(gate.contiguous(), num_expert)
         counts_cpu = counts.cpu()
         pos = pos_buf[: int(counts_cpu.sum())]
     return pos, counts, counts_cpu, slot_to_row

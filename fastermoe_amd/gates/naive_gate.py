@@ -1,7 +1,7 @@
 r"""Top-k of a linear layer (fmoe/gates/naive_gate.py:11-42)."""
-import torch
 import torch.nn as nn
 
+from ..functions import gate_topk
 from .base_gate import BaseGate
 
 
@@ -17,7 +17,9 @@ class NaiveGate(BaseGate):
 
     def forward(self, inp, return_all_scores=False):
         logits = self.gate(inp)
-        top_val, top_idx = torch.topk(logits, k=self.top_k, dim=-1, largest=True, sorted=False)
+        # torch.topk(sorted=False) in the reference; here one kernel that also leaves the expert
+        # histogram and the positions for the layer's routing step (order of the k choices: by logit)
+        top_idx, top_val = gate_topk(logits, self.top_k)
         top_val = top_val.view(-1, self.top_k)
         if return_all_scores:
             return top_idx, top_val, logits

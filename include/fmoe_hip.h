@@ -94,6 +94,35 @@ int fmoe_route_static(const int64_t *gate, int64_t n_slots, int64_t n_expert,
                       int64_t *expert_count, int64_t *pos,
                       int64_t *slot_to_row, void *stream);
 
+/* The gate's top-k, its scores and the routing of fmoe_route in one call: per
+ * token the top_k largest of n_expert logits (ties to the lower expert index,
+ * choices in descending order of the logit),
+ *   topk_idx   [n_tokens, top_k] int64
+ *   topk_score [n_tokens, top_k] (dtype)  score_mode 0: the selected logits
+ *              (what NaiveGate returns, fmoe/gates/naive_gate.py:32-42);
+ *              1: softmax over the top_k selected logits
+ * and, from the per-workgroup histograms the same pass leaves behind,
+ * expert_count / pos / slot_to_row exactly as fmoe_route(topk_idx) gives them.
+ * logits [n_tokens, n_expert] in FMOE_F32 / FMOE_BF16 / FMOE_F16; top_k a power
+ * of two <= 64, n_expert <= 1024 (FMOE_ELIMIT otherwise: use torch.topk and
+ * fmoe_route).  workspace: fmoe_routing_workspace_bytes(n_tokens*top_k, n_expert).
+ * Replaces torch.topk (+ softmax) of fmoe/gates/naive_gate.py:26-42 followed by
+ * count_by_gate, fmoe/functions.py:19-42. */
+int fmoe_gate_topk_route(const void *logits, int64_t n_tokens, int64_t n_expert,
+                         int64_t top_k, int dtype, int score_mode,
+                         int64_t *topk_idx, void *topk_score,
+                         int64_t *expert_count, int64_t *pos,
+                         int64_t *slot_to_row, void *workspace,
+                         int64_t workspace_bytes, void *stream);
+
+/* Gradient of topk_score with respect to the logits, [n_tokens, n_expert]
+ * (zero at experts that were not selected); score is only read in score_mode 1.
+ * Replaces autograd's backward of torch.topk / softmax in the gate. */
+int fmoe_gate_topk_backward(const void *grad_score, const void *score,
+                            const int64_t *topk_idx, void *grad_logits,
+                            int64_t n_tokens, int64_t n_expert, int64_t top_k,
+                            int dtype, int score_mode, void *stream);
+
 /* ---- capacity balancing ------------------------------------------------- */
 
 /* eca[w,e] = share of cap[e] granted to worker w, workers served in ascending

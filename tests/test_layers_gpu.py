@@ -428,14 +428,13 @@ def test_gshard_gate(cap, n, e, device):
     kept = idx >= 0
     assert torch.equal(torch.gather(logits, 1, idx.clamp(min=0))[kept], val[kept])
     # the balance loss of fmoe/gates/gshard_gate.py:23-34 in closed form: both choices of every token counted
-    top_val, top_idx = torch.topk(logits, 2, dim=-1, sorted=False)
+    top_val, top_idx = torch.topk(logits, 2, dim=-1, sorted=True)   # the gate lists a token's choices by logit
     c_e = torch.bincount(top_idx.reshape(-1), minlength=e).double() / n
     m_e = torch.softmax(logits.double(), dim=1).mean(0)
     want_loss = float((c_e * m_e).sum() / e * e * e)
     assert abs(float(gate.get_loss().detach()) - want_loss) <= 1e-5 * want_loss
     assert abs(float(c_e.sum()) - 2.0) < 1e-9
     # first-come-first-kept: what survives the capacity step is the oracle's pruning
-    top_val, top_idx = torch.topk(logits, 2, dim=-1, sorted=False)
     _, _, pruned = orouting.limit_and_prune(top_idx.cpu().numpy(), e, limit)
     survivors = torch.from_numpy(pruned).to(device)
     assert bool(((idx == survivors) | (idx == -1)).all())

@@ -170,3 +170,93 @@ def test_full_size_invariants(device):
     once = fmoe_native.prune_gate_by_capacity(gate, cap.clone(), 256, 1)
     twice = fmoe_native.prune_gate_by_capacity(once, cap.clone(), 256, 1)
     assert torch.equal(once, twice)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,e,k", [
+    (32768, 8, 2),      # the Mixtral-like share: 8 tokens per wave step
+    (8192, 256, 8),     # the fine-grained layer: four logits per lane
+    (16384, 64, 1),     # top-1
+    (16384, 16, 2),
+    (1000, 5, 4),       # experts not a power of two, token count not a multiple of a workgroup's share
+    (77, 1000, 16),     # sixteen logits per lane
+    (3, 2, 2),          # every expert chosen
+    (0, 4, 2),
+])
+def test_gate_topk_route(dtype, n, e, k, device):
+    """fmoe_gate_topk_route against torch.topk (tie-free logits, choices by descending logit), the
+    scores in both modes, and its expert counts / pos / slot_to_row against the CPU oracle run on
+    the SAME index tensor; its backward against autograd through torch.topk and softmax."""
+    from fastermoe_amd import fmoe_native
+    gen = torch.Generator().manual_seed(n + e + k)
+    # distinct values per token, exactly representable in every dtype: consecutive bfloat16 bit patterns
+    # (0.0078 .. 2.6, alternating sign), in a random order per token
+    table = (torch.arange(e, dtype=torch.int16) + 0x3C00).view(torch.bfloat16).float()
+    table = table * (1 - 2 * (torch.arange(e) % 2)).float()
+    base = table[torch.argsort(torch.rand(n, e, generator=gen), dim=1)] if n else torch.zeros(0, e)
+    logits = base.to(dtype).to(device)
+    assert torch.equal(logits.float().cpu(), base)
+    for mode in (0, 1):
+        idx, score, cnt, pos_buf, s2r = fmoe_native.gate_topk_route(logits, k, mode)
+        want_val, want_idx = torch.topk(logits.float(), k, dim=-1, largest=True, sorted=True)
+        assert torch.equal(idx, want_idx)
+        want_score = torch.softmax(want_val, dim=-1) if mode == 1 else want_val
+        if mode == 0:
+            assert torch.equal(score.float(), want_score)
+        else:
+            assert torch.allclose(score.float(), want_score, rtol={torch.float32: 1e-5}.get(dtype, 1e-2), atol=1e-6)
+        ref_pos, ref_cnt = orouting.count_by_gate(idx.cpu().numpy(), e)
+        assert np.array_equal(cnt.cpu().numpy(), ref_cnt)
+        total = int(ref_cnt.sum())
+        assert total == n * k
+        assert np.array_equal(pos_buf[:total].cpu().numpy(), ref_pos)
+        inv = np.full(n * k, -1, dtype=np.int64)
+        inv[ref_pos] = np.arange(total)
+        assert np.array_equal(s2r.cpu().numpy(), inv)
+        if n == 0:
+            continue
+        # backward: d(sum(score * g)) / d(logits)
+        g = torch.randn(n, k, generator=gen).to(dtype).to(device)
+        got = fmoe_native.gate_topk_backward(g, score, idx, e, mode)
+        leaf = logits.float().clone().requires_grad_(True)
+        val, _ = torch.topk(leaf, k, dim=-1, sorted=True)
+        sc = torch.softmax(val, dim=-1) if mode == 1 else val
+        (sc * g.float()).sum().backward()
+        assert torch.allclose(got.float(), leaf.grad, rtol={torch.float32: 1e-5}.get(dtype, 2e-2), atol=1e-2 if dtype != torch.float32 else 1e-6)
+
+
+def test_gate_topk_ties_go_to_the_lower_expert(device):
+    from fastermoe_amd import fmoe_native
+    logits = torch.zeros(9, 6, device=device)
+    logits[:, 4] = 1.0
+    idx, score, cnt, _, _ = fmoe_native.gate_topk_route(logits, 4, 0)
+    assert idx.cpu().tolist() == [[4, 0, 1, 2]] * 9
+    assert cnt.cpu().tolist() == [9, 9, 9, 0, 9, 0]
+    with pytest.raises(ValueError):
+        fmoe_native.gate_topk_route(logits, 3, 0)        # not a power of two: torch.topk + route instead
+
+
+def test_naive_gate_hands_its_routing_to_the_layer(device):
+    """NaiveGate's index tensor carries the routing computed with the top-k; the layer's routing step
+    uses it only for that very tensor, unmodified, and recomputes otherwise."""
+    from fastermoe_amd import functions
+    from fastermoe_amd.gates import NaiveGate
+    torch.manual_seed(8)
+    gate = NaiveGate(32, 8, 1, top_k=2).to(device)
+    x = torch.randn(500, 32, device=device)
+    idx, val = gate(x)
+    assert hasattr(idx, "_fmoe_route")
+    pos_a, cnt_a, cnt_cpu_a, s2r_a = functions._route(idx, 8, 1)
+    fresh = idx.clone()
+    assert not hasattr(fresh, "_fmoe_route")
+    pos_b, cnt_b, _, s2r_b = functions._route(fresh, 8, 1)
+    assert torch.equal(pos_a, pos_b) and torch.equal(cnt_a, cnt_b) and torch.equal(s2r_a, s2r_b)
+    idx[0, 0] = -1                                       # an in-place edit invalidates what rides on the tensor
+    pos_c, cnt_c, _, _ = functions._route(idx, 8, 1)
+    assert int(cnt_c.sum()) == 999
+    # scores are differentiable: the gate's weight gets a gradient through the selected logits
+    idx2, val2 = gate(x)
+    val2.sum().backward()
+    assert gate.gate.weight.grad is not None and torch.isfinite(gate.gate.weight.grad).all()
+    logits = gate.gate(x)
+    assert torch.equal(val2, torch.gather(logits, 1, idx2))
