@@ -956,7 +956,8 @@ float *split_workspace(hipStream_t stream, size_t bytes);
 // compute unit, so `total` tiles run in total / cus rounds and a last, partial round costs as
 // much as a whole one.  When that last round fills at most half the chip, its tiles are split
 // along the contraction into k_split parts (as many as fit the idle units, at most 8, at
-// least 16 slabs each).
+// least 16 slabs each) -- provided that shortens the round by more than the partial sums' round
+// trip through memory costs.
 struct TailSplit {
     int main_tiles, k_split, split_slabs;
 };
@@ -966,7 +967,10 @@ inline TailSplit plan_tail_split(int total, int n_slabs, int cus) {
     if (tail == 0 || tail * 2 > cus) return p;
     int f = std::min(std::min(kMaxSplit, cus / tail), n_slabs / 16);
     if (f < 2) return p;
-    p.split_slabs = (n_slabs + f - 1) / f;
+    const int per_part = (n_slabs + f - 1) / f;
+    // the reduction and the second launch cost about as much as 40 slabs of one tile
+    if (n_slabs - per_part < 40) return p;
+    p.split_slabs = per_part;
     p.k_split = (n_slabs + p.split_slabs - 1) / p.split_slabs;  // no empty part
     p.main_tiles = total - tail;
     return p;

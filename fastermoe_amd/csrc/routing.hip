@@ -269,70 +269,73 @@ __global__ __launch_bounds__(kBlock) void rank_apply_kernel(
 // histogram that the routing scan starts from, in one pass over the logits.
 //
 // A workgroup owns kSlotsPerBlock consecutive (token, choice) slots -- the same slots as
-// workgroup b of rank_apply_kernel -- a wave kSlotsPerWave of them.  A token is worked on by a
-// group of G lanes (G = the power of two at or above n_expert, at most 64), lane g of the group
-// holding logits g, g + G, ...: round j finds the largest remaining logit of the group by
-// xor-shuffles (ties go to the lower expert index), lane j keeps it, and the owner strikes it
-// out.  Lanes 0 .. top_k-1 of a group then hold the token's choices in descending order of the
-// logit; they write index and score, and the wave adds their keys to its private table.
-// score_mode 0: the selected logit itself; 1: softmax over the top_k selected logits.
-template <typename T, int VPL>
+// workgroup b of rank_apply_kernel -- i.e. kSlotsPerBlock / K tokens, 8 / K per thread.  A lane
+// reads its token's row of logits (16 bytes at a time when the rows are aligned) and keeps the K
+// largest in a sorted register list: an insertion is K compare-selects, there is no traffic
+// between lanes, and a later logit only displaces a strictly smaller one, so ties go to the
+// lower expert index.  The choices come out in descending order of the logit.  The wave then
+// adds the selected experts to its private table, one 64-key step per choice.
+// score_mode 0: the selected logit itself; 1: softmax over the K selected logits.
+template <typename T, int K>
 __global__ __launch_bounds__(kBlock) void gate_topk_hist_kernel(
-    const T *__restrict__ logits, int64_t n_tokens, int n_expert, int top_k, int group, int score_mode,
+    const T *__restrict__ logits, int64_t n_tokens, int n_expert, int score_mode, int vector_rows,
     int64_t *__restrict__ topk_idx, T *__restrict__ topk_score, int32_t *__restrict__ block_hist, int nbits) {
     extern __shared__ int32_t bins[];  // [kWavesPerBlock][n_expert]
-    const int wave = threadIdx.x / kWave;
-    int32_t *mine = bins + wave * n_expert;
+    int32_t *mine = bins + (threadIdx.x / kWave) * n_expert;
     for (int e = threadIdx.x; e < kWavesPerBlock * n_expert; e += kBlock) bins[e] = 0;
     __syncthreads();
 
-    const int lane = lane_id();
-    const int g = lane & (group - 1), sub = lane / group;     // lane in its group, group in the wave
-    const int tokens_per_step = kWave / group;
-    const int64_t wave_token0 = ((int64_t)blockIdx.x * kSlotsPerBlock + (int64_t)wave * kSlotsPerWave) / top_k;
-    const int steps = kSlotsPerWave / top_k / tokens_per_step;
+    constexpr int kTokensPerBlock = kSlotsPerBlock / K, kTokensPerThread = kTokensPerBlock / kBlock;
+    constexpr int kVec = 16 / (int)sizeof(T);
     const float kLowest = -__builtin_inff();
-
-    for (int s = 0; s < steps; ++s) {
-        const int64_t token = wave_token0 + (int64_t)s * tokens_per_step + sub;
+    for (int it = 0; it < kTokensPerThread; ++it) {
+        const int64_t token = (int64_t)blockIdx.x * kTokensPerBlock + it * kBlock + threadIdx.x;
         const bool live = token < n_tokens;
-        float v[VPL];
+        float val[K];
+        int idx[K];
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) {
-            const int e = g + i * group;
-            v[i] = (live && e < n_expert) ? (float)logits[token * n_expert + e] : kLowest;
-        }
-        float my_v = kLowest, v_max = 0.f;
-        int my_e = -1;
-        for (int j = 0; j < top_k; ++j) {
-            float best = v[0];
-            int best_e = g;
+        for (int j = 0; j < K; ++j) { val[j] = kLowest; idx[j] = -1; }
+        auto insert = [&](float x, int e) {
 #pragma unroll
-            for (int i = 1; i < VPL; ++i)
-                if (v[i] > best) { best = v[i]; best_e = g + i * group; }
-            for (int m = 1; m < group; m <<= 1) {
-                const float ov = __shfl_xor(best, m, kWave);
-                const int oe = __shfl_xor(best_e, m, kWave);
-                if (ov > best || (ov == best && oe < best_e)) { best = ov; best_e = oe; }
+            for (int j = K - 1; j >= 0; --j) {
+                const bool here = x > val[j];                       // x belongs at or above place j
+                const bool above = j > 0 && x > val[j > 0 ? j - 1 : 0];  // ... above it: place j takes its upper neighbour
+                val[j] = here ? (above ? val[j > 0 ? j - 1 : 0] : x) : val[j];
+                idx[j] = here ? (above ? idx[j > 0 ? j - 1 : 0] : e) : idx[j];
             }
-            if (j == 0) v_max = best;
-            if (g == j) { my_v = best; my_e = best_e; }
+        };
+        if (live) {
+            const T *row = logits + token * n_expert;
+            int e = 0;
+            if (vector_rows) {
+                for (; e + kVec <= n_expert; e += kVec) {
+                    alignas(16) T chunk[kVec];
+                    *(uint4 *)chunk = *(const uint4 *)(row + e);
 #pragma unroll
-            for (int i = 0; i < VPL; ++i)
-                if (g + i * group == best_e) v[i] = kLowest;
+                    for (int c = 0; c < kVec; ++c) insert((float)chunk[c], e + c);
+                }
+            }
+            for (; e < n_expert; ++e) insert((float)row[e], e);
         }
-        const bool chosen = live && g < top_k && my_e >= 0 && my_e < n_expert;
-        float score = my_v;
+        float score[K];
+#pragma unroll
+        for (int j = 0; j < K; ++j) score[j] = val[j];
         if (score_mode == 1) {
-            float ex = chosen ? __expf(my_v - v_max) : 0.f, sum = ex;
-            for (int m = 1; m < group; m <<= 1) sum += __shfl_xor(sum, m, kWave);
-            score = ex / sum;
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < K; ++j) { score[j] = idx[j] >= 0 ? __expf(val[j] - val[0]) : 0.f; sum += score[j]; }
+#pragma unroll
+            for (int j = 0; j < K; ++j) score[j] /= sum;
         }
-        if (live && g < top_k) {
-            topk_idx[token * top_k + g] = chosen ? (int64_t)my_e : -1;
-            topk_score[token * top_k + g] = (T)(chosen ? score : 0.f);
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+            const bool chosen = live && idx[j] >= 0;
+            if (live) {
+                topk_idx[token * K + j] = idx[j];
+                topk_score[token * K + j] = (T)(chosen ? score[j] : 0.f);
+            }
+            wave_bins_add(mine, chosen ? idx[j] : 0, chosen, match_mask(chosen ? idx[j] : 0, chosen, nbits));
         }
-        wave_bins_add(mine, chosen ? my_e : 0, chosen, match_mask(chosen ? my_e : 0, chosen, nbits));
     }
     __syncthreads();
     int32_t *dst = block_hist + (int64_t)blockIdx.x * n_expert;
@@ -620,23 +623,24 @@ namespace {
 template <typename T>
 int launch_gate_topk(const void *logits, int64_t n_tokens, int E, int top_k, int score_mode, int64_t *topk_idx,
                      void *topk_score, int32_t *block_hist, int n_blocks, hipStream_t st) {
-    int group = 1;
-    while (group < E && group < kWave) group <<= 1;
-    const int vpl = (int)ceil_div(E, group);
     const size_t lds = kWavesPerBlock * E * sizeof(int32_t);
     const int nbits = ilog2_ceil(E);
-#define FMOE_GATE_LAUNCH(V)                                                                                       \
+    // rows start on 16-byte boundaries: vector loads
+    const int vector_rows = (E * sizeof(T)) % 16 == 0 && (reinterpret_cast<uintptr_t>(logits) & 15u) == 0;
+#define FMOE_GATE_LAUNCH(KK)                                                                                      \
     do {                                                                                                          \
-        if (int rc = allow_lds((const void *)gate_topk_hist_kernel<T, V>, lds)) return rc;                        \
-        gate_topk_hist_kernel<T, V><<<n_blocks, kBlock, lds, st>>>((const T *)logits, n_tokens, E, top_k, group,  \
-                                                                   score_mode, topk_idx, (T *)topk_score,         \
-                                                                   block_hist, nbits);                            \
+        if (int rc = allow_lds((const void *)gate_topk_hist_kernel<T, KK>, lds)) return rc;                       \
+        gate_topk_hist_kernel<T, KK><<<n_blocks, kBlock, lds, st>>>((const T *)logits, n_tokens, E, score_mode,   \
+                                                                    vector_rows, topk_idx, (T *)topk_score,       \
+                                                                    block_hist, nbits);                           \
     } while (0)
-    if (vpl <= 1) FMOE_GATE_LAUNCH(1);
-    else if (vpl <= 2) FMOE_GATE_LAUNCH(2);
-    else if (vpl <= 4) FMOE_GATE_LAUNCH(4);
-    else if (vpl <= 8) FMOE_GATE_LAUNCH(8);
-    else FMOE_GATE_LAUNCH(16);
+    switch (top_k) {
+        case 1: FMOE_GATE_LAUNCH(1); break;
+        case 2: FMOE_GATE_LAUNCH(2); break;
+        case 4: FMOE_GATE_LAUNCH(4); break;
+        case 8: FMOE_GATE_LAUNCH(8); break;
+        default: return fail(FMOE_ELIMIT, "gate top-k: top_k=%d is not 1, 2, 4 or 8", top_k);
+    }
 #undef FMOE_GATE_LAUNCH
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
@@ -653,10 +657,8 @@ extern "C" int fmoe_gate_topk_route(const void *logits, int64_t n_tokens, int64_
                  (long long)top_k);
     FMOE_REQUIRE(dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16, "fmoe_gate_topk_route: dtype %d", dtype);
     FMOE_REQUIRE(score_mode == 0 || score_mode == 1, "fmoe_gate_topk_route: score_mode %d", score_mode);
-    if (n_expert < 1 || n_expert > 16 * kWave)
-        return fail(FMOE_ELIMIT, "fmoe_gate_topk_route: %lld experts (1..%d)", (long long)n_expert, 16 * kWave);
-    if (top_k > n_expert || top_k > kWave || (top_k & (top_k - 1)) != 0)
-        return fail(FMOE_ELIMIT, "fmoe_gate_topk_route: top_k=%lld must be a power of two, at most 64 and at most n_expert",
+    if (top_k > n_expert || (top_k != 1 && top_k != 2 && top_k != 4 && top_k != 8))
+        return fail(FMOE_ELIMIT, "fmoe_gate_topk_route: top_k=%lld must be 1, 2, 4 or 8 and at most n_expert",
                     (long long)top_k);
     const int64_t n_slots = n_tokens * top_k;
     if (int rc = check_sizes(n_slots, n_expert)) return rc;

@@ -108,7 +108,7 @@ def route(gate, n_expert):
 
 def gate_topk_supported(n_expert, top_k, dtype):
     """Whether :func:`gate_topk_route` takes this gate shape (else: torch.topk and :func:`route`)."""
-    return (1 <= top_k <= min(n_expert, 64) and top_k & (top_k - 1) == 0 and n_expert <= 1024
+    return (top_k in (1, 2, 4, 8) and top_k <= n_expert <= 8192
             and dtype in (torch.float32, torch.bfloat16, torch.float16))
 
 

@@ -49,7 +49,7 @@ class GateTopK(Function):
 
 def gate_topk(logits, top_k, score_mode=0):
     r"""Top-k indices and scores of ``logits [N, E]``: the HIP gate kernel when it takes the shape
-    (CUDA tensor, 16/32-bit floats, ``top_k`` a power of two, at most 1024 experts), ``torch.topk``
+    (CUDA tensor, 16/32-bit floats, ``top_k`` 1, 2, 4 or 8), ``torch.topk``
     otherwise.  ``score_mode`` 0: the selected logits; 1: their softmax over the ``top_k``."""
     if logits.is_cuda and logits.dim() == 2 and fmoe_native.gate_topk_supported(logits.shape[1], top_k, logits.dtype):
         idx, score = GateTopK.apply(logits, top_k, score_mode)

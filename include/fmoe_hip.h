@@ -103,9 +103,8 @@ int fmoe_route_static(const int64_t *gate, int64_t n_slots, int64_t n_expert,
  *              1: softmax over the top_k selected logits
  * and, from the per-workgroup histograms the same pass leaves behind,
  * expert_count / pos / slot_to_row exactly as fmoe_route(topk_idx) gives them.
- * logits [n_tokens, n_expert] in FMOE_F32 / FMOE_BF16 / FMOE_F16; top_k a power
- * of two <= 64, n_expert <= 1024 (FMOE_ELIMIT otherwise: use torch.topk and
- * fmoe_route).  workspace: fmoe_routing_workspace_bytes(n_tokens*top_k, n_expert).
+ * logits [n_tokens, n_expert] in FMOE_F32 / FMOE_BF16 / FMOE_F16; top_k 1, 2, 4
+ * or 8 (FMOE_ELIMIT otherwise: use torch.topk and fmoe_route).  workspace: fmoe_routing_workspace_bytes(n_tokens*top_k, n_expert).
  * Replaces torch.topk (+ softmax) of fmoe/gates/naive_gate.py:26-42 followed by
  * count_by_gate, fmoe/functions.py:19-42. */
 int fmoe_gate_topk_route(const void *logits, int64_t n_tokens, int64_t n_expert,

@@ -225,14 +225,15 @@ def test_gemm_tail_plan_host_logic():
     assert plan(3640, 64) == [3584, 4, 16]             # parts keep at least 16 slabs
     assert plan(3720, 64)[:2] == [3720, 1]             # the last round fills more than half the chip
     assert plan(80, 8)[:2] == [80, 1]                  # contraction too short to split
-    m, f, per = plan(5, 33)
-    assert (m, f) == (0, 2) and per * f >= 33 and per * (f - 1) < 33   # no empty part
+    assert plan(5, 33)[:2] == [5, 1]                   # two parts would save 16 slabs: less than the reduction costs
+    m, f, per = plan(5, 100)
+    assert (m, f) == (0, 6) and per * f >= 100 and per * (f - 1) < 100   # no empty part
     for tiles in range(1, 600, 7):
         for slabs in (1, 15, 16, 31, 32, 100, 224):
             m, f, per = plan(tiles, slabs)
             assert 0 <= m <= tiles and 1 <= f <= 8 and (tiles - m) * f <= 256 or f == 1
             if f > 1:
-                assert per >= 16 and per * f >= slabs and per * (f - 1) < slabs and m % 256 == 0
+                assert per >= 16 and per * f >= slabs and per * (f - 1) < slabs and m % 256 == 0 and slabs - per >= 40
 
 
 def test_reference_import_paths_resolve():

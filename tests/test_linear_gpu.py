@@ -185,11 +185,11 @@ def test_full_depth_bf16_forward_backward(fin, fout, device):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_contraction_split_tail_matches_oracle(dtype, device):
-    """A launch of 2 x 3 + 1 x 3 row/column tiles whose contraction (40 slabs of bf16, 80 of fp32)
+    """A launch of (2 + 1) x 20 row/column tiles whose contraction (80 slabs of bf16, 160 of fp32)
     is split into parts: forward with bias and data-grad, with a ragged contraction tail."""
     g = torch.Generator().manual_seed(23)
     counts = torch.tensor([200, 100])
-    fin, fout = 2560 - 8, 2560 - 24
+    fin, fout = 5120 - 8, 5120 - 24
     x = torch.randn(300, fin, generator=g).to(dtype)
     w = (torch.randn(2, fout, fin, generator=g) / fin ** 0.5).to(dtype)
     b = torch.randn(2, fout, generator=g).to(dtype)

@@ -174,12 +174,13 @@ def test_full_size_invariants(device):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n,e,k", [
-    (32768, 8, 2),      # the Mixtral-like share: 8 tokens per wave step
-    (8192, 256, 8),     # the fine-grained layer: four logits per lane
+    (32768, 8, 2),      # the Mixtral-like share
+    (8192, 256, 8),     # the fine-grained layer
     (16384, 64, 1),     # top-1
     (16384, 16, 2),
     (1000, 5, 4),       # experts not a power of two, token count not a multiple of a workgroup's share
-    (77, 1000, 16),     # sixteen logits per lane
+    (77, 1003, 8),      # rows that do not start on 16-byte boundaries
+    (700, 300, 4),
     (3, 2, 2),          # every expert chosen
     (0, 4, 2),
 ])
