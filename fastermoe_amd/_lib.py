@@ -41,6 +41,8 @@ SIGNATURES = {
     "fmoe_reduce_slots": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "fmoe_index_add_workspace_bytes": (_i64, [_i64, _i64]),
     "fmoe_index_add_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
+    "fmoe_mask_restore": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "fmoe_mask_scale_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_linear_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_linear_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_linear_act_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),

@@ -396,7 +396,102 @@ int permute_zero_unmapped(const int64_t *index, void *out, int64_t n_out, int64_
     return FMOE_OK;
 }
 
+namespace {
+
+// ---- masked tokens: restore the full token order around the rows that went through the experts ----
+// out[t,:] = row[t] >= 0 ? src[row[t],:] : (fill_row[t] >= 0 ? scale[t] * fill[fill_row[t],:] : 0)
+// One workgroup per token row, threads stride over the row (coalesced).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void mask_restore_kernel(
+    const T *__restrict__ src, const int64_t *__restrict__ row, const T *__restrict__ scale,
+    const T *__restrict__ fill, const int64_t *__restrict__ fill_row, T *__restrict__ out, int64_t n_src,
+    int64_t n_fill, int64_t row_elems) {
+    const int64_t t = blockIdx.x;
+    const int64_t r = row[t];
+    T *dst = out + t * row_elems;
+    if (r >= 0 && r < n_src) {
+        const T *s = src + r * row_elems;
+        for (int64_t c = threadIdx.x; c < row_elems; c += kBlock) dst[c] = s[c];
+        return;
+    }
+    const int64_t f = fill_row ? fill_row[t] : -1;
+    if (f >= 0 && f < n_fill) {
+        const float a = scale ? (float)scale[t] : 1.f;
+        const T *s = fill + f * row_elems;
+        for (int64_t c = threadIdx.x; c < row_elems; c += kBlock) dst[c] = (T)(a * (float)s[c]);
+    } else {
+        for (int64_t c = threadIdx.x; c < row_elems; c += kBlock) dst[c] = (T)0.f;
+    }
+}
+
+// grad_scale[t] = masked token with a fill row ? <grad_out[t,:], fill[fill_row[t],:]> : 0, summed in a fixed
+// order: every thread adds its strided share, the 256 partial sums are added in ascending order.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void mask_scale_grad_kernel(
+    const T *__restrict__ grad_out, const int64_t *__restrict__ row, const T *__restrict__ fill,
+    const int64_t *__restrict__ fill_row, T *__restrict__ grad_scale, int64_t n_fill, int64_t row_elems) {
+    __shared__ float part[kBlock];
+    const int64_t t = blockIdx.x;
+    const int64_t f = fill_row[t];
+    float acc = 0.f;
+    const bool masked = row[t] < 0 && f >= 0 && f < n_fill;
+    if (masked) {
+        const T *g = grad_out + t * row_elems, *s = fill + f * row_elems;
+        for (int64_t c = threadIdx.x; c < row_elems; c += kBlock) acc += (float)g[c] * (float)s[c];
+    }
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float sum = 0.f;
+        if (masked)
+            for (int i = 0; i < kBlock; ++i) sum += part[i];
+        grad_scale[t] = (T)sum;
+    }
+}
+
+}  // namespace
 }  // namespace fmoe
+
+extern "C" int fmoe_mask_restore(const void *src, const int64_t *token_to_row, const void *scale, const void *fill,
+                                 const int64_t *fill_row, void *out, int64_t n_tokens, int64_t n_src, int64_t n_fill,
+                                 int64_t row_elems, int dtype, void *stream) {
+    FMOE_REQUIRE(n_tokens >= 0 && n_src >= 0 && n_fill >= 0 && row_elems >= 1, "fmoe_mask_restore: bad sizes");
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_mask_restore: unknown dtype %d", dtype);
+    if (n_tokens == 0) return FMOE_OK;
+    if (n_tokens > (int64_t)INT32_MAX) return fail(FMOE_ELIMIT, "fmoe_mask_restore: %lld tokens", (long long)n_tokens);
+    FMOE_REQUIRE(token_to_row && out && (src || n_src == 0) && ((fill && fill_row) || n_fill == 0),
+                 "fmoe_mask_restore: NULL pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned grid = (unsigned)n_tokens;
+    switch (dtype) {
+        case FMOE_F32: mask_restore_kernel<float><<<grid, kBlock, 0, st>>>((const float *)src, token_to_row, (const float *)scale, (const float *)fill, n_fill ? fill_row : nullptr, (float *)out, n_src, n_fill, row_elems); break;
+        case FMOE_BF16: mask_restore_kernel<__bf16><<<grid, kBlock, 0, st>>>((const __bf16 *)src, token_to_row, (const __bf16 *)scale, (const __bf16 *)fill, n_fill ? fill_row : nullptr, (__bf16 *)out, n_src, n_fill, row_elems); break;
+        case FMOE_F16: mask_restore_kernel<_Float16><<<grid, kBlock, 0, st>>>((const _Float16 *)src, token_to_row, (const _Float16 *)scale, (const _Float16 *)fill, n_fill ? fill_row : nullptr, (_Float16 *)out, n_src, n_fill, row_elems); break;
+        default: mask_restore_kernel<double><<<grid, kBlock, 0, st>>>((const double *)src, token_to_row, (const double *)scale, (const double *)fill, n_fill ? fill_row : nullptr, (double *)out, n_src, n_fill, row_elems); break;
+    }
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_mask_scale_grad(const void *grad_out, const int64_t *token_to_row, const void *fill,
+                                    const int64_t *fill_row, void *grad_scale, int64_t n_tokens, int64_t n_fill,
+                                    int64_t row_elems, int dtype, void *stream) {
+    FMOE_REQUIRE(n_tokens >= 0 && n_fill >= 1 && row_elems >= 1, "fmoe_mask_scale_grad: bad sizes");
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_mask_scale_grad: unknown dtype %d", dtype);
+    if (n_tokens == 0) return FMOE_OK;
+    if (n_tokens > (int64_t)INT32_MAX) return fail(FMOE_ELIMIT, "fmoe_mask_scale_grad: %lld tokens", (long long)n_tokens);
+    FMOE_REQUIRE(grad_out && token_to_row && fill && fill_row && grad_scale, "fmoe_mask_scale_grad: NULL pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned grid = (unsigned)n_tokens;
+    switch (dtype) {
+        case FMOE_F32: mask_scale_grad_kernel<float><<<grid, kBlock, 0, st>>>((const float *)grad_out, token_to_row, (const float *)fill, fill_row, (float *)grad_scale, n_fill, row_elems); break;
+        case FMOE_BF16: mask_scale_grad_kernel<__bf16><<<grid, kBlock, 0, st>>>((const __bf16 *)grad_out, token_to_row, (const __bf16 *)fill, fill_row, (__bf16 *)grad_scale, n_fill, row_elems); break;
+        case FMOE_F16: mask_scale_grad_kernel<_Float16><<<grid, kBlock, 0, st>>>((const _Float16 *)grad_out, token_to_row, (const _Float16 *)fill, fill_row, (_Float16 *)grad_scale, n_fill, row_elems); break;
+        default: return fail(FMOE_EINVAL, "fmoe_mask_scale_grad: float32, bfloat16 or float16 only");
+    }
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
 
 extern "C" int fmoe_gather_rows(const void *inp, const int64_t *index, void *out, int64_t n_out, int64_t n_inp,
                                 int64_t row_elems, int dtype, void *stream) {

@@ -244,6 +244,38 @@ def index_add_rows(inp, index, n_out):
     return out
 
 
+def mask_restore(src, token_to_row, scale, fill, fill_row, n_tokens):
+    """out[t] = src[token_to_row[t]] for kept tokens, scale[t] * fill[fill_row[t]] for masked tokens
+    that have a fill row, zero otherwise.  ``fill`` may be ``None`` (no fill rows at all)."""
+    dt = _rows("src", src)
+    _dev("token_to_row", token_to_row, torch.int64)
+    n_fill = 0
+    if fill is not None:
+        _dev("fill", fill, src.dtype)
+        _dev("fill_row", fill_row, torch.int64)
+        n_fill = fill.shape[0]
+        if scale is not None:
+            _dev("scale", scale, src.dtype)
+    out = torch.empty(n_tokens, src.shape[1], dtype=src.dtype, device=src.device)
+    with torch.cuda.device(src.device):
+        check(_lib.load().fmoe_mask_restore(_ptr(src), _ptr(token_to_row), _ptr(scale if fill is not None else None),
+                                            _ptr(fill), _ptr(fill_row if fill is not None else None), _ptr(out),
+                                            n_tokens, src.shape[0], n_fill, src.shape[1], dt, _stream(src)))
+    return out
+
+
+def mask_scale_grad(grad_out, token_to_row, fill, fill_row):
+    """Per-token dot product of the output gradient with the token's fill row (masked tokens only)."""
+    dt = _rows("grad_out", grad_out)
+    _dev("fill", fill, grad_out.dtype)
+    grad_scale = torch.empty(grad_out.shape[0], dtype=grad_out.dtype, device=grad_out.device)
+    with torch.cuda.device(grad_out.device):
+        check(_lib.load().fmoe_mask_scale_grad(_ptr(grad_out), _ptr(token_to_row), _ptr(fill), _ptr(fill_row),
+                                               _ptr(grad_scale), grad_out.shape[0], fill.shape[0], grad_out.shape[1],
+                                               dt, _stream(grad_out)))
+    return grad_scale
+
+
 # ---- score-weighted combine ---------------------------------------------------------
 
 def combine_forward(x, score, n_tokens, top_k):

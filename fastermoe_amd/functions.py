@@ -280,6 +280,63 @@ class MOEGatherCombine(Function):
         return grad_rows, None, grad_score.view(score_shape), None, None
 
 
+def mask_index(mask):
+    r"""For FMoE's ``mask`` (fmoe/layers.py:288-293): ``(keep_idx, token_to_row)`` -- the indices of
+    the tokens whose mask is 0 (what ``inp[mask == 0]`` selects, here in descending token order)
+    and, per token, its row among the kept ones (-1 for masked tokens).  One routing call with a
+    single "expert" and one device-to-host read (the number of kept tokens), no boolean indexing."""
+    with torch.no_grad():
+        key = (mask.reshape(-1) != 0).to(torch.int64).neg_()        # 0: keep, -1: masked
+        counts, pos_buf, token_to_row = fmoe_native.route(key, 1)
+        keep_idx = pos_buf[: int(counts.cpu()[0])]
+    return keep_idx, token_to_row
+
+
+class MaskSelect(Function):
+    r"""``rows[keep_idx]``: the rows of the kept tokens (``inp[mask == 0, :]``, fmoe/layers.py:292);
+    the backward puts the gradient rows back and leaves zero rows for masked tokens."""
+
+    @staticmethod
+    def forward(ctx, rows, keep_idx, token_to_row):
+        ctx.save_for_backward(token_to_row)
+        return fmoe_native.gather_rows(rows.contiguous(), keep_idx)
+
+    @staticmethod
+    def backward(ctx, grad_rows):
+        (token_to_row,) = ctx.saved_tensors
+        return fmoe_native.gather_rows(grad_rows.contiguous(), token_to_row), None, None
+
+
+class MaskRestore(Function):
+    r"""Back to the full token order (fmoe/layers.py:305-317, with the combine of :322 already
+    applied to the kept tokens): ``out[t] = kept[token_to_row[t]]`` for kept tokens and
+    ``scale[t] * fill[fill_row[t]]`` for a masked token whose mask value has a ``mask_dict`` entry
+    (``scale`` = the sum of the token's gate scores, since every one of its ``top_k`` slots holds
+    the same ``mask_dict`` value), zero rows otherwise.  ``fill`` may be ``None``."""
+
+    @staticmethod
+    def forward(ctx, kept, keep_idx, token_to_row, scale, fill, fill_row):
+        ctx.save_for_backward(keep_idx, token_to_row, scale, fill, fill_row)
+        return fmoe_native.mask_restore(kept.contiguous(), token_to_row, scale, fill, fill_row, token_to_row.numel())
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        keep_idx, token_to_row, scale, fill, fill_row = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        grad_kept = fmoe_native.gather_rows(grad_out, keep_idx)
+        grad_scale = grad_fill = None
+        if fill is not None and scale is not None and ctx.needs_input_grad[3]:
+            grad_scale = fmoe_native.mask_scale_grad(grad_out, token_to_row, fill, fill_row)
+        if fill is not None and ctx.needs_input_grad[4]:
+            # a mask_dict value that is trained: rare, plain torch
+            masked = (token_to_row < 0) & (fill_row >= 0)
+            w = scale.float() if scale is not None else torch.ones_like(fill_row, dtype=torch.float32)
+            contrib = (grad_out.float() * (w * masked).unsqueeze(1))
+            grad_fill = torch.zeros(fill.shape, dtype=torch.float32, device=fill.device).index_add_(
+                0, fill_row.clamp(min=0), contrib).to(fill.dtype)
+        return grad_kept, None, None, grad_scale, grad_fill, None
+
+
 class AllGather(Function):
     r"""fmoe/functions.py:333-349 (model-parallel group); one worker only."""
 

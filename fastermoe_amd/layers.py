@@ -6,8 +6,9 @@ import os
 import torch
 import torch.nn as nn
 
-from .functions import (AllGather, MOECache, MOECombine, MOEGather, MOEGatherCombine, MOELinear, MOEScatter, Slice,
-                        _prepare_forward_ex, ensure_comm)
+from . import fmoe_native
+from .functions import (AllGather, MaskRestore, MaskSelect, MOECache, MOECombine, MOEGather, MOEGatherCombine,
+                        MOELinear, MOEScatter, Slice, _prepare_forward_ex, ensure_comm, mask_index)
 from .gates import NaiveGate
 
 
@@ -189,6 +190,52 @@ class FMoE(nn.Module):
                 mark_module_parallel_comm(self.experts, expert_dp_comm)
         mark_module_parallel_comm(self.gate, "moe")
 
+    def _mask_kernels_apply(self, inp, gate_top_k_idx, gate_score):
+        """The index-kernel form of the mask path needs GPU tensors, one gate index and one score per
+        (token, k) pair and mask_dict values that are one row of d_model each."""
+        n = inp.shape[0]
+        return (inp.is_cuda and inp.is_floating_point() and inp.dtype != torch.float64
+                and torch.is_tensor(gate_score) and gate_score.dtype == inp.dtype
+                and gate_top_k_idx.numel() == gate_score.numel() == n * self.top_k
+                and self.mask.numel() == n
+                and all(torch.is_tensor(v) and v.numel() == self.d_model for v in self.mask_dict.values())
+                and os.environ.get("FMOE_MASK_KERNELS", "1") != "0")
+
+    def _forward_masked(self, inp, gate_top_k_idx, gate_score):
+        r"""fmoe/layers.py:288-322 without boolean indexing: the kept tokens' rows, gate indices and
+        scores are gathered over an index built by one routing call, go through the experts and the
+        folded combine, and one kernel restores the token order, writing
+        ``sum_j score[t,j] * mask_dict[mask[t]]`` for the masked tokens (all ``top_k`` slots of a
+        masked token hold the same ``mask_dict`` row)."""
+        n, k, d = inp.shape[0], self.top_k, self.d_model
+        mask = self.mask.view(-1).to(inp.device)
+        keep_idx, token_to_row = mask_index(mask)
+        score = gate_score.reshape(n, k)
+        inp_k = MaskSelect.apply(inp, keep_idx, token_to_row)
+        score_k = MaskSelect.apply(score, keep_idx, token_to_row)
+        idx_k = fmoe_native.gather_rows(gate_top_k_idx.reshape(n, k).contiguous().view(torch.float64),
+                                        keep_idx).view(torch.int64)
+        if os.environ.get("FMOE_FOLD_COMBINE", "1") != "0":
+            y_k, _ = _fmoe_general_global_forward(
+                inp_k, idx_k, self.expert_fn, self.policy_fn, self.experts, self.num_expert, self.world_size,
+                self.experts_fused, self.enable_fuse, score_k)
+        else:
+            rows, _ = _fmoe_general_global_forward(
+                inp_k, idx_k, self.expert_fn, self.policy_fn, self.experts, self.num_expert, self.world_size,
+                self.experts_fused, self.enable_fuse)
+            y_k = MOECombine.apply(rows.reshape(-1, d), score_k.reshape(-1, 1, k), inp_k.shape[0], k)
+        # which mask_dict row a masked token takes (-1: its mask value has no entry -> zero row)
+        keys = sorted(int(key) for key in self.mask_dict)
+        fill = fill_row = scale = None
+        if keys:
+            fill = torch.cat([self.mask_dict[key].reshape(1, d) for key in keys]).to(device=inp.device, dtype=inp.dtype)
+            lut = torch.full((max(keys) + 2,), -1, dtype=torch.int64, device=inp.device)
+            lut[torch.tensor(keys, device=inp.device)] = torch.arange(len(keys), device=inp.device)
+            lut[0] = -1
+            fill_row = lut[mask.clamp(min=0, max=max(keys) + 1)]
+            scale = score.sum(dim=-1).contiguous()
+        return MaskRestore.apply(y_k, keep_idx, token_to_row, scale, fill, fill_row)
+
     def forward(self, inp):
         r"""Gate, route through the experts, and combine each token's ``top_k``
         expert outputs with the gate scores (fmoe/layers.py:272-326)."""
@@ -202,6 +249,11 @@ class FMoE(nn.Module):
             self.gate_hook(gate_top_k_idx, gate_score, None)
 
         masked = self.mask is not None and self.mask_dict is not None
+        if masked and self._mask_kernels_apply(inp, gate_top_k_idx, gate_score):
+            x = self._forward_masked(inp, gate_top_k_idx, gate_score)
+            if self.mp_size > 1:
+                x = AllGather.apply(x, self.mp_rank, self.mp_size, self.mp_group)
+            return x
         if masked:
             mask = self.mask.view(-1)
             inp = inp[mask == 0, :]

@@ -173,6 +173,31 @@ int fmoe_index_add_rows(const void *inp, const int64_t *index, void *out,
                         int dtype, void *workspace, int64_t workspace_bytes,
                         void *stream);
 
+/* Masked tokens (FMoE's mask / mask_dict, fmoe/layers.py:288-319).  The kept
+ * tokens are selected with fmoe_gather_rows over an index of the tokens whose
+ * mask is 0 (fmoe_route with one "expert" yields that index and its inverse);
+ * after the experts, the full token order is restored in one pass:
+ *   out[t,:] = token_to_row[t] >= 0 ? src[token_to_row[t],:]
+ *            : fill_row[t] >= 0    ? scale[t] * fill[fill_row[t],:]   (scale NULL: 1)
+ *            : 0
+ * src [n_src,row], fill [n_fill,row] (the mask_dict values), fill_row [n_tokens]
+ * int64 (which mask_dict value a masked token takes, -1: none), scale
+ * [n_tokens] (the sum of the token's gate scores when the combine is folded in).
+ * Replaces the zeros() + boolean-index assignments of fmoe/layers.py:309-317. */
+int fmoe_mask_restore(const void *src, const int64_t *token_to_row,
+                      const void *scale, const void *fill,
+                      const int64_t *fill_row, void *out, int64_t n_tokens,
+                      int64_t n_src, int64_t n_fill, int64_t row_elems,
+                      int dtype, void *stream);
+
+/* Gradient of fmoe_mask_restore with respect to scale: grad_scale[t] =
+ * <grad_out[t,:], fill[fill_row[t],:]> for masked tokens with a fill row, else
+ * 0 (autograd of the bmm over the restored rows, fmoe/layers.py:321-322). */
+int fmoe_mask_scale_grad(const void *grad_out, const int64_t *token_to_row,
+                         const void *fill, const int64_t *fill_row,
+                         void *grad_scale, int64_t n_tokens, int64_t n_fill,
+                         int64_t row_elems, int dtype, void *stream);
+
 /* ---- score-weighted combination of the top-k expert outputs ------------- */
 
 /* out[t,:] = sum_{j<top_k} score[t,j] * x[t*top_k+j,:], accumulated in fp32.

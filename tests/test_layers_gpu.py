@@ -492,6 +492,42 @@ def test_zero_and_noisy_gate_and_mask(device):
     assert torch.allclose(ym[mask == 1], 7.0 * score[mask == 1].expand(-1, 16))
 
 
+@pytest.mark.parametrize("fuse", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_masked_tokens_index_kernels_match_boolean_indexing(fuse, dtype, device, monkeypatch):
+    """mask / mask_dict (fmoe/layers.py:288-319): the index-kernel path (select kept tokens, experts,
+    folded combine, one restore pass) against the reference's boolean-index formulation
+    (FMOE_MASK_KERNELS=0): output, input gradient, expert gradients and the gate's gradient, which
+    also flows through the masked tokens' scores.  Mask values: 0 keep, 1 and 2 replaced by their
+    mask_dict rows, 5 without an entry (zero rows); a CPU mask as in tests/test_zero.py."""
+    torch.manual_seed(21)
+    n, d, h, e, k = 301, 64, 96, 4, 2
+    mask = torch.zeros(n, dtype=torch.long)
+    mask[torch.randperm(n)[:120]] = torch.tensor([1, 2, 5]).repeat(40)
+    fills = {1: torch.randn(d).to(dtype).to(device), 2: torch.randn(1, d).to(dtype).to(device)}
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, mask=mask, mask_dict=fills)
+    moe.enable_fuse = fuse
+    moe = moe.to(dtype).to(device)
+    x = torch.randn(n, d).to(dtype).to(device)
+    results = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("FMOE_MASK_KERNELS", flag)
+        moe.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        (out.float() * torch.linspace(-1, 1, d, device=device)).mean().backward()
+        results.append([out, xi.grad, moe.gate.gate.weight.grad.clone()] + [p.grad.clone() for p in moe.experts.parameters()])
+    tol = TOL[dtype] * (1 if dtype == torch.bfloat16 else 10)
+    for a, b in zip(*results):
+        assert rel_err(a, b) <= tol, rel_err(a, b)
+    out = results[0][0]
+    assert torch.count_nonzero(out[(mask == 5).to(device)]) == 0
+    with torch.no_grad():
+        score = moe.gate(x)[1]
+    want = score.float().sum(-1, keepdim=True)[(mask == 1).to(device)] * fills[1].float()
+    assert torch.allclose(out[(mask == 1).to(device)].float(), want, rtol=2e-2 if dtype == torch.bfloat16 else 1e-5, atol=1e-5)
+
+
 def test_gate_hook_and_state_dict(device):
     seen = {}
     moe = fmoe.FMoETransformerMLP(num_expert=2, d_model=8, d_hidden=16, top_k=2,
@@ -583,3 +619,51 @@ def test_fused_gelu_epilogue_accuracy(dtype, device):
     got_gb1 = gb1.float().view(-1)[:d]
     assert ((got_gb1 - want_gb1).abs() <= 4 * step * want_gb1.abs() + 0.05 * step * n).all()
     assert torch.count_nonzero(gb1.float().view(-1)[d:]) == 0
+
+
+def test_noisy_gate_against_the_published_definitions(device):
+    """NoisyGate (Shazeer et al. 2017): evaluation mode against top-k + softmax + hard counts; training
+    mode with the noise replayed from the seed, the smooth load against kth_excluding computed by
+    brute force (sort the noisy logits without component i) for every (token, expert)."""
+    torch.manual_seed(13)
+    n, d, e, k = 40, 16, 6, 2
+    gate = NoisyGate(d, e, 1, top_k=k).to(device)
+    x = torch.randn(n, d, device=device)
+
+    def cv2(v):
+        return v.var() / (v.mean() ** 2 + 1e-10)
+
+    gate.eval()
+    idx, score = gate(x)
+    clean = x @ gate.w_gate
+    want_val, want_idx = torch.topk(clean, k, dim=1, sorted=True)
+    assert torch.equal(idx.view(n, k), want_idx)
+    assert torch.allclose(score.view(n, k), torch.softmax(want_val, dim=1), rtol=1e-5, atol=1e-6)
+    imp = torch.zeros(e, device=device).index_add(0, want_idx.reshape(-1), torch.softmax(want_val, dim=1).reshape(-1))
+    load = torch.bincount(want_idx.reshape(-1), minlength=e).float()
+    assert torch.allclose(gate.get_loss(), cv2(imp) + cv2(load), rtol=1e-4)
+    assert hasattr(idx, "_fmoe_route")
+
+    gate.train()
+    torch.manual_seed(99)
+    idx, score = gate(x)
+    torch.manual_seed(99)
+    noise = torch.randn_like(clean)
+    std = torch.nn.functional.softplus(x @ gate.w_noise) + 1e-2
+    noisy = clean + noise * std
+    want_val, want_idx = torch.topk(noisy, k, dim=1, sorted=True)
+    assert torch.equal(idx.view(n, k), want_idx)
+    assert torch.allclose(score.view(n, k), torch.softmax(want_val, dim=1), rtol=1e-5, atol=1e-6)
+    prob = torch.zeros(n, e, dtype=torch.float64)
+    nz, cl, sd = noisy.detach().double().cpu(), clean.detach().double().cpu(), std.detach().double().cpu()
+    for t in range(n):
+        for i in range(e):
+            others = torch.cat([nz[t, :i], nz[t, i + 1:]]).sort(descending=True).values
+            z = (cl[t, i] - others[k - 1]) / sd[t, i]
+            prob[t, i] = 0.5 * (1 + math.erf(float(z) / math.sqrt(2)))
+    imp = torch.zeros(e, device=device).index_add(0, want_idx.reshape(-1), torch.softmax(want_val, dim=1).reshape(-1))
+    want_loss = cv2(imp.detach().double().cpu()) + cv2(prob.sum(0))
+    loss = gate.get_loss()
+    assert abs(float(loss.detach()) - float(want_loss)) <= 1e-4 * float(want_loss)
+    loss.backward()
+    assert gate.w_noise.grad is not None and torch.isfinite(gate.w_noise.grad).all()
