@@ -52,7 +52,8 @@ SIGNATURES = {
     "fmoe_fused_mlp_forward": (_int, [ctypes.POINTER(MlpParams), _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                       _vp, _vp, _vp, _vp, _vp, _int, _vp]),
     "fmoe_fused_mlp_backward": (_int, [ctypes.POINTER(MlpParams), _vp, _vp, _vp, _vp, _i64, _i64, _i64,
-                                       _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
+                                       _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
+    "fmoe_fused_scatter_in_loader": (_int, [ctypes.POINTER(MlpParams), _vp, _i64]),
     "fmoe_combine_forward": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_combine_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_gather_combine_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),

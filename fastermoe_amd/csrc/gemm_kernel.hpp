@@ -154,6 +154,12 @@ struct GemmParams {
     int32_t activation;
     int32_t accumulate_first;  // ragged-K: expert 0 of the table adds to C
     int32_t epilogue;          // Epilogue, read by the any-shape kernel only
+    // Ragged rows with a [row][contraction] row operand (the forward product) only: when q_row_index
+    // is set, row r of the expert-sorted order is read from row q_row_index[r] / q_index_div of Q
+    // (the token matrix, q_total_rows rows) instead of row r -- the local scatter happens in the
+    // loader and the sorted copy of the input is never written.
+    const int64_t *q_row_index;
+    int64_t q_index_div, q_total_rows;
     // Ragged rows only.  The tiles beyond the last whole round of the chip (tiles main_tiles ..
     // total_tiles - 1 of the logical order) can be split along the contraction: k_split
     // workgroups compute split_slabs slabs each and leave their fp32 accumulators in split_ws;
@@ -259,12 +265,16 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     const T *Qb;
     T *Cb;
     int p_valid, q_valid, K;
+    int q_row0 = 0;
+    const bool gather_q = RAGGED == kRaggedRows && QSHAPE == kKC && prm.q_row_index != nullptr;
+    int64_t q_gather_bytes = 0;  // extent of the gathered matrix past this part's first contraction element
     int64_t aux_off;  // offset of this tile's origin inside C (and aux)
     if (RAGGED == kRaggedRows) {
         const int row0 = seg_lo + (mt - prm.tab.tile[ei]) * BM;
+        q_row0 = row0;
         q_valid = min(BM, seg_hi - row0);
         K = prm.k_extent;
-        Qb = (const T *)prm.Q + (int64_t)row0 * prm.ldq;
+        Qb = (const T *)prm.Q + (gather_q ? (int64_t)0 : (int64_t)row0 * prm.ldq);
         const T *Pe = (const T *)prm.P + (int64_t)expert * prm.p_expert_stride;
         Pb = (PSHAPE == kKC) ? Pe + (int64_t)n0 * prm.ldp : Pe + n0;
         aux_off = (int64_t)row0 * prm.ldc + n0;
@@ -272,6 +282,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             const int k_begin = split_part * prm.split_slabs * BKE;
             K = max(0, min(K - k_begin, prm.split_slabs * BKE));
             Qb += (QSHAPE == kKC) ? (int64_t)k_begin : (int64_t)k_begin * prm.ldq;
+            q_gather_bytes = -(int64_t)k_begin * (int64_t)sizeof(T);
             Pb += (PSHAPE == kKC) ? (int64_t)k_begin : (int64_t)k_begin * prm.ldp;
         }
     } else {
@@ -353,11 +364,26 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     if (QSHAPE == kKC) {
         const int r = t >> 3;
         q_kc_chunk = (t & 7) ^ swz(r);
+        if (gather_q) {
+            // the resource covers the whole token matrix (less than 2 GiB, checked by the host) from this
+            // part's first contraction element on; a row index outside it reads as zeros
+            q_gather_bytes += prm.q_total_rows * prm.ldq * (int64_t)sizeof(T);
 #pragma unroll
-        for (int it = 0; it < NQ; ++it)
-            q_voff[it] = (it * kRowsPerPass + r < q_valid)
-                             ? (uint32_t)(((int64_t)(it * kRowsPerPass + r) * prm.ldq + q_kc_chunk * CE) * sizeof(T))
-                             : kOutOfRange;
+            for (int it = 0; it < NQ; ++it) {
+                const int row = it * kRowsPerPass + r;
+                int64_t src = -1;
+                if (row < q_valid && t < kLoaders) src = prm.q_row_index[q_row0 + row] / prm.q_index_div;
+                q_voff[it] = (src >= 0 && src < prm.q_total_rows)
+                                 ? (uint32_t)((src * prm.ldq + q_kc_chunk * CE) * (int64_t)sizeof(T))
+                                 : kOutOfRange;
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < NQ; ++it)
+                q_voff[it] = (it * kRowsPerPass + r < q_valid)
+                                 ? (uint32_t)(((int64_t)(it * kRowsPerPass + r) * prm.ldq + q_kc_chunk * CE) * sizeof(T))
+                                 : kOutOfRange;
+        }
     } else {
         const int kk = t / Q_CPR;
 #pragma unroll
@@ -400,12 +426,14 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // the chunk is dropped when it lies past K.  MC: the resource starts at contraction row
     // k0 and is exactly as long as the rows that remain, so rows past K read as zero.
     auto issue_part = [&](auto shape_tag, const T *tile, int64_t ld, int kc_chunk, const uint32_t *voff, auto n_tag, int k0,
-                          uint32_t lds_off, int it_lo = 0, int it_hi = 1 << 20) {
+                          uint32_t lds_off, int it_lo = 0, int it_hi = 1 << 20, int64_t kc_extent = (int64_t)1 << 40) {
         constexpr int SHAPE = decltype(shape_tag)::value;
         constexpr int N = decltype(n_tag)::value;
         const int k_left = K - k0;  // <= 0 past the end: everything reads as zero
         const T *origin = (SHAPE == kKC) ? tile + k0 : tile + (int64_t)k0 * ld;
-        int64_t bytes = (SHAPE == kKC) ? (int64_t)kOutOfRange : (int64_t)k_left * ld * (int64_t)sizeof(T);
+        // KC: the rows of a tile lie within 2 GiB of its origin; gathered rows within kc_extent bytes of the matrix
+        int64_t bytes = (SHAPE == kKC) ? kc_extent - (int64_t)k0 * (int64_t)sizeof(T)
+                                       : (int64_t)k_left * ld * (int64_t)sizeof(T);
         bytes = bytes < 0 ? 0 : (bytes > (int64_t)kOutOfRange ? (int64_t)kOutOfRange : bytes);
         const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(origin), 0, (int)bytes, kRsrcFlags);
         // sign bit of (k_left - 1 - first k of the chunk): set exactly when the chunk starts past K
@@ -427,7 +455,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     };
     auto issue_q = [&](int k0, int buf) {
         issue_part(std::integral_constant<int, QSHAPE>{}, Qb, prm.ldq, q_kc_chunk, q_voff, std::integral_constant<int, NQ>{}, k0,
-                   (uint32_t)(Q_BASE + buf * Q_BYTES));
+                   (uint32_t)(Q_BASE + buf * Q_BYTES), 0, 1 << 20, gather_q ? q_gather_bytes : (int64_t)1 << 40);
     };
 
     // Data-grad with the activation derivative, 16-bit types: the tile of saved

@@ -326,6 +326,12 @@ float *split_workspace(hipStream_t stream, size_t bytes) {
 
 }  // namespace gemm
 
+bool linear_forward_can_gather(const LinearForwardArgs &a) {
+    if (a.dtype == FMOE_F64 || dtype_bytes(a.dtype) == 0) return false;
+    if (!is_fast(a.dtype, {a.x, a.w, a.y, a.aux, a.bias}, {a.in_feat, a.out_feat})) return false;
+    return a.x_total_rows >= 0 && a.x_total_rows * a.in_feat * (int64_t)dtype_bytes(a.dtype) < ((int64_t)1 << 31);
+}
+
 int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
                            int64_t row_hi, hipStream_t stream) {
     int64_t total;
@@ -336,6 +342,8 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
     FMOE_REQUIRE(a.x && a.w && a.y, "linear_forward: NULL tensor");
     const Plan plan = plan_rows(counts, n_expert, row_lo, row_hi);
     const bool fast = is_fast(a.dtype, {a.x, a.w, a.y, a.aux, a.bias}, {a.in_feat, a.out_feat});
+    FMOE_REQUIRE(a.x_row_index == nullptr || linear_forward_can_gather(a),
+                 "linear_forward: rows cannot be gathered in the loader for this shape");
     const int block_m = pick_rows_height(counts, n_expert, row_lo, row_hi, a.out_feat);
     for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
         const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
@@ -344,6 +352,7 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
         fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, block_m);
         prm.profile_class = kProfGemmFwd; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
         prm.P = a.w; prm.Q = a.x; prm.C = a.y; prm.bias = a.bias; prm.aux = a.aux;
+        prm.q_row_index = a.x_row_index; prm.q_index_div = a.x_index_div; prm.q_total_rows = a.x_total_rows;
         prm.ldp = a.in_feat; prm.ldq = a.in_feat; prm.ldc = a.out_feat;
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.bias_expert_stride = a.out_feat;

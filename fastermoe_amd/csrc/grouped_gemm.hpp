@@ -25,14 +25,22 @@ struct SegmentTable {
 };
 
 struct LinearForwardArgs {
-    const void *x;      // [rows, in]
+    const void *x;      // [rows, in]; with x_row_index: the token matrix [x_total_rows, in]
     const void *w;      // [E, out, in]
     const void *bias;   // [E, out] or null
     void *y;            // [rows, out]
     void *aux;          // [rows, out] pre-activation copy (kEpiBiasAct) or null
     int64_t in_feat, out_feat;
     int dtype, epilogue, activation;
+    // optional: sorted row r is read from row x_row_index[r] / x_index_div of x (local scatter in the
+    // loader); only honoured where linear_forward_can_gather() says so
+    const int64_t *x_row_index = nullptr;
+    int64_t x_index_div = 1, x_total_rows = 0;
 };
+
+// Whether the forward product can read its rows through an index: the MFMA path (aligned pointers,
+// feature sizes that are multiples of 16 bytes) and a token matrix of less than 2 GiB.
+bool linear_forward_can_gather(const LinearForwardArgs &a);
 
 struct LinearDgradArgs {
     const void *gy;     // [rows, out]

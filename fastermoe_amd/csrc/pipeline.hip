@@ -34,7 +34,7 @@ constexpr int kMaxChunks = 32;
 struct DeviceLanes {
     bool ready = false;
     hipStream_t in = nullptr, compute = nullptr, out = nullptr;
-    hipEvent_t fork = nullptr, join_in = nullptr, join_compute = nullptr, join_out = nullptr;
+    hipEvent_t fork = nullptr, join_in = nullptr, join_compute = nullptr, join_out = nullptr, regather = nullptr;
     hipEvent_t in_ready[kMaxChunks] = {};
     hipEvent_t out_ready[kMaxChunks] = {};
 };
@@ -52,7 +52,7 @@ int get_lanes(DeviceLanes **out) {
         FMOE_HIP_CHECK(hipStreamCreateWithFlags(&l.in, hipStreamNonBlocking));
         FMOE_HIP_CHECK(hipStreamCreateWithFlags(&l.compute, hipStreamNonBlocking));
         FMOE_HIP_CHECK(hipStreamCreateWithFlags(&l.out, hipStreamNonBlocking));
-        hipEvent_t *single[] = {&l.fork, &l.join_in, &l.join_compute, &l.join_out};
+        hipEvent_t *single[] = {&l.fork, &l.join_in, &l.join_compute, &l.join_out, &l.regather};
         for (hipEvent_t *e : single) FMOE_HIP_CHECK(hipEventCreateWithFlags(e, hipEventDisableTiming));
         for (int c = 0; c < kMaxChunks; ++c) {
             FMOE_HIP_CHECK(hipEventCreateWithFlags(&l.in_ready[c], hipEventDisableTiming));
@@ -189,6 +189,14 @@ extern "C" int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t
     return FMOE_OK;
 }
 
+extern "C" int fmoe_fused_scatter_in_loader(const fmoe_mlp_params *p, const void *inp, int64_t n_tokens) {
+    if (p == nullptr || inp == nullptr || n_tokens < 0) return 0;
+    // the output pointers only matter for their alignment; torch allocations are 256-byte aligned
+    LinearForwardArgs probe{inp, p->w1, p->b1, nullptr, nullptr, p->d_model, p->d_hidden, p->dtype, kEpiBiasAct,
+                            p->activation, nullptr, 1, n_tokens};
+    return linear_forward_can_gather(probe) ? 1 : 0;
+}
+
 extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp, const int64_t *pos,
                                       const int64_t *slot_to_row, const int64_t *expert_count_host,
                                       int64_t n_tokens, int64_t top_k, int64_t n_rows, void *buf_in,
@@ -199,8 +207,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     const int64_t n_slots = n_tokens * top_k;
     if (n_slots == 0) return FMOE_OK;
     FMOE_REQUIRE(slot_to_row || !out, "fmoe_fused_mlp_forward: NULL slot_to_row");
-    FMOE_REQUIRE(n_rows == 0 || (inp && pos && buf_in && buf_mid && buf_out),
-                 "fmoe_fused_mlp_forward: NULL buffer");
+    FMOE_REQUIRE(n_rows == 0 || (inp && pos && buf_mid && buf_out), "fmoe_fused_mlp_forward: NULL buffer");
     const int dt = p->dtype;
     const int64_t d = p->d_model, h = p->d_hidden, E = p->n_expert;
     hipStream_t caller = (hipStream_t)stream;
@@ -214,7 +221,14 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     if (out && n_rows < n_slots)
         if (int rc = permute_zero_unmapped(slot_to_row, out, n_slots, d, dt, l->out)) return rc;
 
-    for (int c = 0; c < n_chunks; ++c) {
+    // The first GEMM reads the token rows through pos in its loader where it can; buf_in is then
+    // neither written nor needed (the caller passes NULL).
+    LinearForwardArgs probe{inp, p->w1, p->b1, buf_mid, buf_pre, d, h, dt, kEpiBiasAct, p->activation, pos, top_k, n_tokens};
+    const bool in_loader = buf_in == nullptr;
+    FMOE_REQUIRE(!in_loader || n_rows == 0 || linear_forward_can_gather(probe),
+                 "fmoe_fused_mlp_forward: buf_in is NULL but this shape needs the scattered copy "
+                 "(ask fmoe_fused_scatter_in_loader first)");
+    for (int c = 0; c < n_chunks && !in_loader; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         // permute-in: buf_in[r] = inp[pos[r] / top_k]
@@ -225,9 +239,9 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
-        FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
+        if (!in_loader) FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
         LinearForwardArgs f1{buf_in, p->w1, p->b1, buf_mid, buf_pre, d, h, dt, kEpiBiasAct, p->activation};
-        if (int rc = grouped_linear_forward(f1, expert_count_host, E, lo, hi, l->compute)) return rc;
+        if (int rc = grouped_linear_forward(in_loader ? probe : f1, expert_count_host, E, lo, hi, l->compute)) return rc;
         LinearForwardArgs f2{buf_mid, p->w2, p->b2, buf_out, nullptr, h, d, dt, kEpiStore, FMOE_ACT_NONE};
         if (int rc = grouped_linear_forward(f2, expert_count_host, E, lo, hi, l->compute)) return rc;
         FMOE_HIP_CHECK(hipEventRecord(l->out_ready[c], l->compute));
@@ -245,8 +259,8 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
 
 extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *grad_out, const int64_t *pos,
                                        const int64_t *slot_to_row, const int64_t *expert_count_host,
-                                       int64_t n_tokens, int64_t top_k, int64_t n_rows, const void *buf_in,
-                                       const void *buf_pre, const void *buf_mid, void *g_out, void *g_mid,
+                                       int64_t n_tokens, int64_t top_k, int64_t n_rows, const void *inp,
+                                       void *buf_in, const void *buf_pre, const void *buf_mid, void *g_out, void *g_mid,
                                        void *g_in, void *grad_inp, void *grad_w1, void *grad_b1, void *grad_w2,
                                        void *grad_b2, int n_chunks, void *stream) {
     if (int rc = check_common("fmoe_fused_mlp_backward", p, expert_count_host, n_tokens, top_k, n_rows, n_chunks))
@@ -267,6 +281,14 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     int64_t bounds[kMaxChunks + 1];
     chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, compute_units_or_default(), bounds);
 
+    // A forward that read the token rows in its loader kept no sorted copy of the input; the first
+    // linear's weight gradient contracts over sorted rows, so the copy is made now (inp != NULL),
+    // on the permute-in lane, long before that product runs.
+    if (inp != nullptr && n_rows > 0) {
+        FMOE_REQUIRE(pos != nullptr, "fmoe_fused_mlp_backward: pos is NULL");
+        if (int rc = permute_gather_rows(inp, pos, top_k, buf_in, n_rows, n_tokens, d, dt, l->in)) return rc;
+    }
+    FMOE_HIP_CHECK(hipEventRecord(l->regather, l->in));
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
@@ -302,6 +324,7 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     // (the bias gradients come out of the weight-gradient kernel's first column tiles).
     LinearWgradArgs w2{g_out, buf_mid, grad_w2, grad_b2, h, d, dt};
     if (int rc = grouped_linear_wgrad(w2, expert_count_host, E, 0, n_rows, true, l->compute)) return rc;
+    FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->regather, 0));
     LinearWgradArgs w1{g_mid, buf_in, grad_w1, grad_b1, d, h, dt};
     if (int rc = grouped_linear_wgrad(w1, expert_count_host, E, 0, n_rows, true, l->compute)) return rc;
     return join_lanes(l, caller);

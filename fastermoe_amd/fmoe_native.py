@@ -481,9 +481,11 @@ def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k
                       slot_order=True):
     """scatter -> Linear -> activation -> Linear -> gather as one pipelined call.
     Returns ``(out [N*top_k, d], buf_in, buf_pre or None, buf_mid)``; the three
-    buffers are what the backward needs.  With ``slot_order=False`` the copy to
-    slot order is skipped and ``out`` is the experts' output in expert-sorted
-    order, ``[n_rows, d]``."""
+    buffers are what the backward needs.  ``buf_in`` is ``None`` when the first GEMM read the
+    token rows through ``pos`` in its loader (no sorted copy of the input exists; the backward
+    makes one from ``inp``).  With ``slot_order=False`` the copy to slot order is skipped and
+    ``out`` is the experts' output in expert-sorted order, ``[n_rows, d]``."""
+    import os
     prm, n_expert, d_model, d_hidden = _mlp_params(w1, b1, w2, b2, activation)
     _dev("inp", inp, w1.dtype)
     _dev("pos", pos, torch.int64)
@@ -495,11 +497,15 @@ def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k
         raise ValueError("slot_to_row must have n_tokens * top_k entries")
     cnt = _host_counts("expert_count", expert_count, n_expert)
     new = lambda r, c: torch.empty(r, c, dtype=inp.dtype, device=inp.device)
-    buf_in, buf_mid, buf_out = new(n_rows, d_model), new(n_rows, d_hidden), new(n_rows, d_model)
+    lib = _lib.load()
+    in_loader = (os.environ.get("FMOE_FOLD_SCATTER", "1") != "0" and n_rows > 0
+                 and lib.fmoe_fused_scatter_in_loader(ctypes.byref(prm), _ptr(inp), n_tokens) == 1)
+    buf_in = None if in_loader else new(n_rows, d_model)
+    buf_mid, buf_out = new(n_rows, d_hidden), new(n_rows, d_model)
     buf_pre = new(n_rows, d_hidden) if activation == _lib.ACT_GELU else None
     out = new(n_tokens * top_k, d_model) if slot_order else None
     with torch.cuda.device(inp.device):
-        check(_lib.load().fmoe_fused_mlp_forward(
+        check(lib.fmoe_fused_mlp_forward(
             ctypes.byref(prm), _ptr(inp), _ptr(pos), _ptr(slot_to_row), ctypes.c_void_p(cnt.data_ptr()),
             n_tokens, top_k, n_rows, _ptr(buf_in), _ptr(buf_pre), _ptr(buf_mid), _ptr(buf_out), _ptr(out),
             n_chunks, _stream(inp)))
@@ -507,12 +513,13 @@ def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k
 
 
 def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid,
-                       n_tokens, top_k, activation, n_chunks, slot_order=True):
+                       n_tokens, top_k, activation, n_chunks, slot_order=True, inp=None):
     """Backward of :func:`fused_mlp_forward`.  Returns
     ``(grad_inp, grad_w1, grad_b1, grad_w2, grad_b2)`` (bias grads ``None``
     without biases).  For ReLU the post-activation buffer doubles as the
     pre-activation (same sign pattern).  With ``slot_order=False``, ``grad_out``
-    is already in expert-sorted order, ``[n_rows, d]``."""
+    is already in expert-sorted order, ``[n_rows, d]``.  ``buf_in=None``: the forward kept no
+    sorted copy of the input; it is rebuilt here from ``inp`` ``[n_tokens, d]``."""
     prm, n_expert, d_model, d_hidden = _mlp_params(w1, b1, w2, b2, activation)
     _dev("grad_out", grad_out, w1.dtype)
     n_rows = pos.numel()
@@ -523,6 +530,12 @@ def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2,
     pre = buf_pre if buf_pre is not None else buf_mid
     dev, dty = grad_out.device, grad_out.dtype
     new = lambda *s: torch.empty(*s, dtype=dty, device=dev)
+    regather = buf_in is None
+    if regather:
+        if inp is None:
+            raise ValueError("fused_mlp_backward: neither buf_in nor inp")
+        _dev("inp", inp, w1.dtype)
+        buf_in = new(n_rows, d_model)
     g_out = new(n_rows, d_model) if slot_order else grad_out
     g_mid, g_in = new(n_rows, d_hidden), new(n_rows, d_model)
     grad_inp = new(n_tokens, d_model)
@@ -533,7 +546,8 @@ def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2,
         check(_lib.load().fmoe_fused_mlp_backward(
             ctypes.byref(prm), _ptr(grad_out if slot_order else None), _ptr(pos), _ptr(slot_to_row),
             ctypes.c_void_p(cnt.data_ptr()),
-            n_tokens, top_k, n_rows, _ptr(buf_in), _ptr(pre), _ptr(buf_mid), _ptr(g_out), _ptr(g_mid), _ptr(g_in),
+            n_tokens, top_k, n_rows, _ptr(inp if regather else None), _ptr(buf_in), _ptr(pre), _ptr(buf_mid),
+            _ptr(g_out), _ptr(g_mid), _ptr(g_in),
             _ptr(grad_inp), _ptr(grad_w1), _ptr(grad_b1), _ptr(grad_w2), _ptr(grad_b2), n_chunks,
             _stream(grad_out)))
     return grad_inp, grad_w1, grad_b1, grad_w2, grad_b2
@@ -565,9 +579,11 @@ def fused_forward(input_buf, params, local_expert_count, global_expert_count, st
     w1, b1, w2, b2 = _unpack_params(params, has_bias)
     rows = input_buf.shape[0]
     ident = torch.arange(rows, dtype=torch.int64, device=input_buf.device)
-    out, buf_in, _pre, buf_mid = fused_mlp_forward(input_buf.contiguous(), ident, ident, global_expert_count,
+    input_buf = input_buf.contiguous()
+    out, buf_in, _pre, buf_mid = fused_mlp_forward(input_buf, ident, ident, global_expert_count,
                                                    w1, b1, w2, b2, 1, _lib.ACT_RELU, _fuse_chunks())
-    return [out, buf_in, buf_mid, out]
+    # global_input_buf of the reference: with the identity permutation it is the input itself
+    return [out, buf_in if buf_in is not None else input_buf, buf_mid, out]
 
 
 def fused_backward(input_buf, params, middle_buf, output_buf, grad_out, local_expert_count,

@@ -43,20 +43,24 @@ class _FusedExpertMLP(Function):
     @staticmethod
     def forward(ctx, inp, w1, b1, w2, b2, pos, slot_to_row, expert_count, top_k, activation, n_chunks,
                 slot_order=True):
+        inp = inp.contiguous()
         out, buf_in, buf_pre, buf_mid = fmoe_native.fused_mlp_forward(
-            inp.contiguous(), pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k, activation, n_chunks,
-            slot_order)
-        ctx.save_for_backward(pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid)
-        ctx.moe_args = inp.shape[0], top_k, activation, n_chunks, slot_order
+            inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k, activation, n_chunks, slot_order)
+        # without a sorted copy of the input (the first GEMM gathered the rows itself) the backward
+        # rebuilds one from the input, which autograd keeps alive anyway
+        ctx.save_for_backward(pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in if buf_in is not None else inp,
+                              buf_pre, buf_mid)
+        ctx.moe_args = inp.shape[0], top_k, activation, n_chunks, slot_order, buf_in is None
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid = ctx.saved_tensors
-        n_tokens, top_k, activation, n_chunks, slot_order = ctx.moe_args
+        n_tokens, top_k, activation, n_chunks, slot_order, regather = ctx.moe_args
         grad_inp, gw1, gb1, gw2, gb2 = fmoe_native.fused_mlp_backward(
-            grad_out.contiguous(), pos, slot_to_row, expert_count, w1, b1, w2, b2, buf_in, buf_pre, buf_mid,
-            n_tokens, top_k, activation, n_chunks, slot_order)
+            grad_out.contiguous(), pos, slot_to_row, expert_count, w1, b1, w2, b2,
+            None if regather else buf_in, buf_pre, buf_mid,
+            n_tokens, top_k, activation, n_chunks, slot_order, inp=buf_in if regather else None)
         return grad_inp, gw1, gb1, gw2, gb2, None, None, None, None, None, None, None
 
 

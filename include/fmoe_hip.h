@@ -326,7 +326,10 @@ int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert,
  *   inp        [n_tokens, d_model]
  *   pos        [n_rows] int64   flat slot of every expert-sorted row
  *   slot_to_row[n_tokens*top_k] int64 (inverse of pos, -1 = dropped)
- *   buf_in     [n_rows, d_model]   scattered input  (kept for backward)
+ *   buf_in     [n_rows, d_model]   scattered input  (kept for backward); NULL: the
+ *              first GEMM reads the token rows through pos in its loader and no
+ *              sorted copy of the input is made (only where
+ *              fmoe_fused_scatter_in_loader says so)
  *   buf_pre    [n_rows, d_hidden]  pre-activation   (kept for backward)
  *   buf_mid    [n_rows, d_hidden]  post-activation  (kept for backward)
  *   buf_out    [n_rows, d_model]   expert output
@@ -336,6 +339,12 @@ int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert,
  * Replaces fmoe_cuda_fused_forward_impl at one worker,
  * cuda/fused_compute.cuh:250-388 (fmoe_cuda.fused_forward) together with the
  * _local_scatter/_local_gather around it, fmoe/fused_functions.py:22-32. */
+/* 1 when fmoe_fused_mlp_forward can take buf_in = NULL for this layer and input
+ * (MFMA path: 16-byte aligned pointers, feature sizes that are multiples of 16
+ * bytes; token matrix below 2 GiB), else 0.  Host only. */
+int fmoe_fused_scatter_in_loader(const fmoe_mlp_params *p, const void *inp,
+                                 int64_t n_tokens);
+
 int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
                            const int64_t *pos, const int64_t *slot_to_row,
                            const int64_t *expert_count_host, int64_t n_tokens,
@@ -345,7 +354,9 @@ int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
 
 /* Backward of the same pipeline.  grad_out [n_tokens*top_k, d_model]; NULL: the
  * caller has already put the gradient rows in expert-sorted order into g_out
- * (e.g. with fmoe_gather_combine_backward).
+ * (e.g. with fmoe_gather_combine_backward).  inp != NULL: the forward kept no
+ * sorted copy of the input (buf_in = NULL there); buf_in is then scratch that
+ * this call fills from inp [n_tokens, d_model] on its permute lane.
  * Scratch (caller-allocated): g_out [n_rows,d_model], g_mid [n_rows,d_hidden],
  * g_in [n_rows,d_model].  Results: grad_inp [n_tokens,d_model], grad_w1/2,
  * grad_b1/2 (bias grads may be NULL).  The data gradients run chunk by chunk;
@@ -357,8 +368,9 @@ int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
 int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *grad_out,
                             const int64_t *pos, const int64_t *slot_to_row,
                             const int64_t *expert_count_host, int64_t n_tokens,
-                            int64_t top_k, int64_t n_rows, const void *buf_in,
-                            const void *buf_pre, const void *buf_mid,
+                            int64_t top_k, int64_t n_rows, const void *inp,
+                            void *buf_in, const void *buf_pre,
+                            const void *buf_mid,
                             void *g_out, void *g_mid, void *g_in,
                             void *grad_inp, void *grad_w1, void *grad_b1,
                             void *grad_w2, void *grad_b2, int n_chunks,

@@ -613,7 +613,7 @@ def test_fused_gelu_epilogue_accuracy(dtype, device):
     torch.nn.functional.gelu(pre_leaf).sum().backward()
     grad_inp, gw1, gb1, gw2, gb2 = fmoe_native.fused_mlp_backward(
         torch.ones(n, d, device=device, dtype=dtype), pos, pos.clone(), cnt, w1, b1, w2, None, buf_in, buf_pre,
-        buf_mid, n, 1, _lib.ACT_GELU, 1)
+        buf_mid, n, 1, _lib.ACT_GELU, 1, inp=x)
     # gb1[j] = sum_rows g_mid[:, j] with g_mid = (ones . W2)[:, j] * GELU'(pre[:, j]); W2 picks the first d units
     want_gb1 = (pre_leaf.grad[:, :d]).sum(0)
     got_gb1 = gb1.float().view(-1)[:d]
@@ -667,3 +667,40 @@ def test_noisy_gate_against_the_published_definitions(device):
     assert abs(float(loss.detach()) - float(want_loss)) <= 1e-4 * float(want_loss)
     loss.backward()
     assert gate.w_noise.grad is not None and torch.isfinite(gate.w_noise.grad).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_scatter_in_the_gemm_loader_equals_the_scattered_copy(dtype, device, monkeypatch):
+    """The fused pipeline's first GEMM reads the token rows through pos in its loader
+    (FMOE_FOLD_SCATTER=0: from a scattered copy made by the permute stage, as
+    fmoe/fused_functions.py:22 does).  Same bits out of the forward -- the products and their order
+    are identical -- and the same gradients; drops, an empty expert, ragged tiles, several chunks."""
+    from fastermoe_amd import fmoe_native
+    monkeypatch.setenv("FMOE_FUSE_GRAN", "3")
+    torch.manual_seed(77)
+    n, d, h, e, k = 700, 128, 320, 5, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe.enable_fuse = True
+    moe = moe.to(dtype).to(device)
+    x = torch.randn(n, d).to(dtype).to(device)
+    idx = torch.randint(-1, e - 1, (n, k), device=device)
+    score = torch.rand(n, k, device=device).to(dtype)
+    moe.gate.forward = lambda inp: (idx, score)
+    results = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("FMOE_FOLD_SCATTER", flag)
+        moe.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        out.float().mean().backward()
+        results.append([out, xi.grad] + [p.grad.clone() for p in moe.experts.parameters()])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    # and the low-level call really runs without a scattered copy
+    cnt, pos_buf, s2r = fmoe_native.route(idx, e)
+    pos = pos_buf[: int(cnt.sum())]
+    ex = moe.experts
+    monkeypatch.setenv("FMOE_FOLD_SCATTER", "1")
+    _, buf_in, _, _ = fmoe_native.fused_mlp_forward(x, pos, s2r, cnt.cpu(), ex.htoh4.weight, ex.htoh4.bias,
+                                                    ex.h4toh.weight, ex.h4toh.bias, k, 2, 3)
+    assert buf_in is None
