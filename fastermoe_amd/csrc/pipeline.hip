@@ -16,9 +16,9 @@
 // permute-out stage), and grad_out = NULL in the backward when it has already
 // written the gradient rows in sorted order (no permute-in stage).
 //
-// All streams use the default priority.  Events are created once per device and
-// reused; a call therefore must not overlap another call of this library's fused
-// entry points on the same device from a different host thread.
+// All streams use the default priority.  Streams and events are created once per
+// device and reused; host threads that call the fused entry points on the same
+// device are serialised by a per-device mutex while they enqueue.
 #include "grouped_gemm.hpp"
 #include "permute.hpp"
 
@@ -41,6 +41,9 @@ struct DeviceLanes {
 
 std::mutex g_lanes_mutex;
 DeviceLanes g_lanes[16];
+// One fused call at a time enqueues on a device's lanes: host threads that call the fused entry points
+// on the same device are serialised here (their work is still ordered by their own streams' fork/join).
+std::mutex g_enqueue_mutex[16];
 
 int get_lanes(DeviceLanes **out) {
     int dev = 0;
@@ -213,6 +216,7 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     hipStream_t caller = (hipStream_t)stream;
     DeviceLanes *l;
     if (int rc = get_lanes(&l)) return rc;
+    std::lock_guard<std::mutex> enqueue_lock(g_enqueue_mutex[l - g_lanes]);
     if (int rc = fork_lanes(l, caller)) return rc;
     int64_t bounds[kMaxChunks + 1];
     chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, compute_units_or_default(), bounds);
@@ -277,6 +281,7 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     hipStream_t caller = (hipStream_t)stream;
     DeviceLanes *l;
     if (int rc = get_lanes(&l)) return rc;
+    std::lock_guard<std::mutex> enqueue_lock(g_enqueue_mutex[l - g_lanes]);
     if (int rc = fork_lanes(l, caller)) return rc;
     int64_t bounds[kMaxChunks + 1];
     chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, compute_units_or_default(), bounds);
