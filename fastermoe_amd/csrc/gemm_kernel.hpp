@@ -19,11 +19,16 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Waves of a workgroup along C's rows and columns: 4 x 2 (512 threads, two waves per SIMD,
-// 64 x 128 per wave), so that the matrix pipe stays fed while one wave of a SIMD sits at
-// the barrier or waits for LDS.
-constexpr int kWavesM = 4, kWavesN = 2;
-constexpr int kThreads = 64 * kWavesM * kWavesN;
+// Waves of a workgroup along C's rows and columns.  Tiles 256 columns wide: 4 x 2 (512 threads,
+// two waves per SIMD, 64 x 128 or 32 x 128 per wave), so that the matrix pipe stays fed while one
+// wave of a SIMD sits at the barrier or waits for LDS; the workgroup takes the whole LDS of a
+// compute unit.  Tiles of 128 x 128: 2 x 2 (256 threads, 64 x 64 per wave) and half the LDS, so two
+// workgroups share a compute unit and one's first loads and epilogue run under the other's main
+// loop -- for launches whose tiles are short (few slabs) or few.
+constexpr int kWavesN = 2;
+constexpr int waves_m_of(int bn) { return bn == 128 ? 2 : 4; }
+constexpr int threads_of(int bn) { return 64 * waves_m_of(bn) * kWavesN; }
+constexpr int kThreads = threads_of(256);  // the any-shape kernels' workgroup size
 // The first kLoadWaves waves of a workgroup request the slabs.  The SIMD issues from its
 // oldest wave first, so with two waves per SIMD the younger one falls behind; leaving the
 // loads (which can block at a full load queue) to the older waves evens the two out.
@@ -31,7 +36,7 @@ constexpr int kLoadWaves = 4;
 constexpr int kLoaders = 64 * kLoadWaves;
 constexpr int kRowsPerPass = kLoaders / 8;  // KC slabs: rows covered by one 16-byte load of every loading thread
 constexpr int kSlabBytes = 128;  // contraction bytes per row per slab
-constexpr int kGroupM = 8;       // row tiles that share a column tile consecutively
+constexpr int kGroupM = 4;       // row tiles that share a column tile consecutively (an XCD then runs 4 x 8 tiles at a time)
 
 enum Shape { kKC = 0, kMC = 1 };
 enum Ragged { kRaggedRows = 0, kRaggedK = 1 };
@@ -168,7 +173,7 @@ struct GemmParams {
     // the epilogue.  k_split == 1: main_tiles == total_tiles.
     float *split_ws;
     int32_t main_tiles, k_split, split_slabs, fixup;
-    int32_t block_m;           // host only: tile height the segment table was built for (256 or 128)
+    int32_t block_m, block_n;  // host only: tile height the segment table was built for (256 or 128) and tile width
     int32_t profile_class;     // host only: ProfileClass of this launch
     double profile_work;       // host only: flop of this launch
     SegmentTable tab;
@@ -187,8 +192,11 @@ template <typename T> __device__ __forceinline__ int mc_swz(int k) {
 
 // ---- the kernel ---------------------------------------------------------------
 template <typename T, int BM, int BN, int PSHAPE, int QSHAPE, int RAGGED, int EPI>
-__global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
+__global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const GemmParams prm) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
+    constexpr int kWavesM = waves_m_of(BN), kWaves = kWavesM * kWavesN;
+    constexpr int kThreads = threads_of(BN);
+    static_assert(kWaves >= kLoadWaves && (kWaves & (kWaves - 1)) == 0, "wave layout");
     constexpr int CE = Elem<T>::kPerChunk;           // elements per 16-byte chunk
     constexpr int BKE = kSlabBytes / (int)sizeof(T); // elements per slab row
     constexpr int WM = BM / kWavesM, WN = BN / kWavesN;  // wave tile
@@ -217,7 +225,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
             int L;
             const int main_grid = (prm.main_tiles + 7) & ~7;
             if (fixup) {
-                tail_index = blockIdx.x >> 3;  // eight one-wave workgroups per tail tile
+                tail_index = blockIdx.x / kWaves;  // one one-wave workgroup per wave of a tail tile
                 L = prm.main_tiles + tail_index;
             } else if ((int)blockIdx.x < main_grid) {
                 const int per_xcd = main_grid >> 3;
@@ -297,8 +305,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     Cb = (T *)prm.C + aux_off;
 
     const int t = threadIdx.x;
-    // a fixup launch runs one wave per workgroup; it stands in for wave blockIdx.x % 8 of the tile's workgroup
-    const int lane = t & 63, wave = fixup ? (int)(blockIdx.x & 7) : t >> 6;
+    // a fixup launch runs one wave per workgroup; it stands in for wave blockIdx.x % kWaves of the tile's workgroup
+    const int lane = t & 63, wave = fixup ? (int)(blockIdx.x % kWaves) : t >> 6;
     const int lb = lane & (MB - 1), hq = lane / MB;  // row inside an MFMA block, contraction chunk inside a step
     const int wave_m0 = (wave / kWavesN) * WM, wave_n0 = (wave % kWavesN) * WN;
 
@@ -784,30 +792,32 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // (32 x 32 blocks: g = 0..3, hq = 0..1; 16 x 16 blocks: g = 0, hq = 0..3): a lane owns
     // runs of 4 consecutive columns in many different rows, which written straight to
     // memory would touch one cache line per row and store.  Instead every wave passes its sub-tile
-    // through a private LDS staging area of [WM rows][256 B + 16 B pad] and moves it
-    // between LDS and memory with 16-byte accesses that cover whole 256-byte row pieces
-    // (4 rows per wave instruction).  Tiles that are read in the epilogue (the saved
+    // through a private LDS staging area of [WM rows][256 B + 16 B pad] (128 B + 16 B for the
+    // 64-column wave tiles of 16-bit types) and moves it between LDS and memory with 16-byte
+    // accesses that cover whole row pieces (4 or 8 rows per wave instruction).  Tiles that are read in the epilogue (the saved
     // pre-activation, or C itself when accumulating) come in through the same area.
     if constexpr (RAGGED == kRaggedK && QSHAPE == kMC) {
         if (want_bias) __syncthreads();  // the bias reduction used the start of LDS
     }
-    constexpr int kStgRow = 256 + 16;            // bytes; the pad spreads rows over the banks
-    constexpr int CPP = 256 / (int)sizeof(T);    // C columns per pass through the staging area
+    constexpr int kPieceBytes = WN * (int)sizeof(T) < 256 ? WN * (int)sizeof(T) : 256;  // row piece moved per pass
+    constexpr int kStgRow = kPieceBytes + 16;    // bytes; the pad spreads rows over the banks
+    constexpr int CPP = kPieceBytes / (int)sizeof(T);  // C columns per pass through the staging area
     constexpr int XPP = CPP / MB;                // MFMA block columns per pass
     constexpr int NPASS = WN / CPP;
     unsigned char *stg = smem + (fixup ? 0 : wave) * (WM * kStgRow);
     const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride + n0 : nullptr;
     T *aux = prm.aux ? (T *)prm.aux + aux_off : nullptr;
     const bool accumulate = (RAGGED == kRaggedK) && prm.accumulate_first && ei == 0;
-    const int io_r = lane >> 4, io_c = lane & 15;  // coalesced side: 4 rows x 16 chunks per instruction
+    constexpr int kPieceChunks = kPieceBytes / 16, kIoRows = 64 / kPieceChunks;
+    const int io_r = lane / kPieceChunks, io_c = lane % kPieceChunks;  // coalesced side: kIoRows rows x whole pieces per instruction
 
     auto lds_sync = [&]() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup"); __builtin_amdgcn_wave_barrier(); };
 
     // memory -> staging (rows/columns outside the tile read as zero)
     auto stage_in = [&](const T *src, int col_base) {
 #pragma unroll
-        for (int i = 0; i < WM / 4; ++i) {
-            const int r = i * 4 + io_r;
+        for (int i = 0; i < WM / kIoRows; ++i) {
+            const int r = i * kIoRows + io_r;
             u32x4 v = u32x4{0, 0, 0, 0};
             if (wave_m0 + r < q_valid && col_base + io_c * CE < p_valid)
                 v = *(const u32x4 *)(src + (int64_t)(wave_m0 + r) * prm.ldc + col_base + io_c * CE);
@@ -817,8 +827,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // staging -> memory
     auto stage_out = [&](T *dst, int col_base) {
 #pragma unroll
-        for (int i = 0; i < WM / 4; ++i) {
-            const int r = i * 4 + io_r;
+        for (int i = 0; i < WM / kIoRows; ++i) {
+            const int r = i * kIoRows + io_r;
             const u32x4 v = *(const u32x4 *)(stg + r * kStgRow + io_c * 16);
             if (wave_m0 + r < q_valid && col_base + io_c * CE < p_valid)
                 *(u32x4 *)(dst + (int64_t)(wave_m0 + r) * prm.ldc + col_base + io_c * CE) = v;
@@ -1006,9 +1016,11 @@ inline TailSplit plan_tail_split(int total, int n_slabs, int cus) {
 
 template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI>
 int launch_tiles(GemmParams &prm, hipStream_t stream) {
-    // three P and two Q slab buffers, or the epilogue's staging area (one [rows][256 B + 16 B] block per wave)
+    constexpr int kWavesM = waves_m_of(BN), kThreads = threads_of(BN);
+    // three P and two Q slab buffers, or the epilogue's staging area (one [rows][row piece + 16 B] block per wave)
     constexpr int smem_loop = (3 * BN + 2 * BM) * kSlabBytes;
-    constexpr int smem_wave_epi = (BM / kWavesM) * (256 + 16);
+    constexpr int wave_cols_bytes = BN / kWavesN * (int)sizeof(T);
+    constexpr int smem_wave_epi = (BM / kWavesM) * ((wave_cols_bytes < 256 ? wave_cols_bytes : 256) + 16);
     constexpr int smem_epi = kWavesM * kWavesN * smem_wave_epi;
     constexpr int smem = smem_loop > smem_epi ? smem_loop : smem_epi;
     // the opt-in to more than 64 KiB of dynamic LDS is per device (and per kernel instantiation)
@@ -1032,7 +1044,9 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
     if (RG == kRaggedRows) {
         constexpr int BKE = kSlabBytes / (int)sizeof(T);
         const int n_slabs = (prm.k_extent + BKE - 1) / BKE;
-        const TailSplit ts = plan_tail_split(prm.total_tiles, n_slabs, device_compute_units());
+        // (two 128 x 128 workgroups share a compute unit: their launches are not split)
+        const TailSplit ts = BN == 256 ? plan_tail_split(prm.total_tiles, n_slabs, device_compute_units())
+                                       : TailSplit{prm.total_tiles, 1, n_slabs};
         if (ts.k_split > 1) {
             const int tail = prm.total_tiles - ts.main_tiles;
             float *ws = split_workspace(stream, (size_t)tail * ts.k_split * BM * BN * sizeof(float));
@@ -1069,13 +1083,12 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
     return FMOE_OK;
 }
 
-// Tile counts, then the launch for the requested epilogue.  prm.block_m (256 or 128,
-// chosen by the host from the segment lengths) is the tile height; the width is 256.
+// Tile counts, then the launch for the requested epilogue.  prm.block_m x prm.block_n (256 x 256,
+// 128 x 256 or 128 x 128, chosen by the host from the segment lengths) is the tile.
 // EPI_MASK lists the epilogues a product can be asked for, so that only those kernels
 // are built.
-template <typename T, int BM, int PS, int QS, int RG, int EPI_MASK>
+template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI_MASK>
 int launch_for_height(GemmParams &prm, int epi, hipStream_t stream) {
-    constexpr int BN = 256;
     prm.tiles_n = (int)ceil_div(prm.n_cols, BN);
     int64_t total;
     if (RG == kRaggedRows) {
@@ -1098,9 +1111,10 @@ int launch_for_height(GemmParams &prm, int epi, hipStream_t stream) {
 
 template <typename T, int PS, int QS, int RG, int EPI_MASK>
 int launch_by_epilogue(GemmParams &prm, int epi, hipStream_t stream) {
-    if (prm.block_m == 128) return launch_for_height<T, 128, PS, QS, RG, EPI_MASK>(prm, epi, stream);
-    if (prm.block_m == 256) return launch_for_height<T, 256, PS, QS, RG, EPI_MASK>(prm, epi, stream);
-    return fail(FMOE_EINVAL, "tile height %d is not built", prm.block_m);
+    if (prm.block_m == 128 && prm.block_n == 128) return launch_for_height<T, 128, 128, PS, QS, RG, EPI_MASK>(prm, epi, stream);
+    if (prm.block_m == 128 && prm.block_n == 256) return launch_for_height<T, 128, 256, PS, QS, RG, EPI_MASK>(prm, epi, stream);
+    if (prm.block_m == 256 && prm.block_n == 256) return launch_for_height<T, 256, 256, PS, QS, RG, EPI_MASK>(prm, epi, stream);
+    return fail(FMOE_EINVAL, "tile %d x %d is not built", prm.block_m, prm.block_n);
 }
 
 }  // namespace gemm

@@ -20,6 +20,8 @@
 #include "profile.hpp"
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <initializer_list>
 #include <mutex>
 #include <vector>
@@ -123,31 +125,41 @@ void fill_table(SegmentTable *tab, const int64_t *counts, int e0, int e1, int64_
     tab->tile[tab->n] = tiles;
 }
 
-// Tile height for a ragged-rows product: 256 unless that gives too few tiles to occupy
-// the chip; then 128.  (Halving the height to cut the padding of short segments was
-// measured and lost: with ~256 rows per expert the product is bound by streaming the
-// weights, which a lower tile re-reads twice as often.)
-int pick_rows_height(const int64_t *counts, int64_t n_expert, int64_t row_lo, int64_t row_hi, int64_t n_cols) {
-    int64_t start = 0, rows = 0, padded = 0;
+// Tile of a launch.  256 x 256 (one workgroup per compute unit) unless that gives too few tiles
+// to occupy the chip: then 128 x 256, and when even those number fewer than two per compute unit,
+// 128 x 128 (two workgroups per compute unit).  (Lower tiles to cut the padding of short segments
+// were measured and lost: with ~256 rows per expert the product is bound by streaming the weights,
+// which a lower tile re-reads more often; and 128 x 128 tiles lose a quarter of the rate of large
+// launches, because they read each operand from L2 and LDS more often per flop.)
+// FMOE_GEMM_TILE=256x256|128x256|128x128 forces one shape (for tests and measurements).
+struct TileShape {
+    int bm, bn;
+};
+TileShape pick_tile(int64_t tiles_256) {
+    if (const char *e = getenv("FMOE_GEMM_TILE")) {
+        if (!strcmp(e, "256x256")) return {256, 256};
+        if (!strcmp(e, "128x256")) return {128, 256};
+        if (!strcmp(e, "128x128")) return {128, 128};
+    }
+    if (tiles_256 >= 512) return {256, 256};
+    return tiles_256 >= 256 ? TileShape{128, 256} : TileShape{128, 128};
+}
+
+// ragged rows: tiles_256 counts every expert's rows rounded up to whole 256-row tiles
+TileShape pick_rows_tile(const int64_t *counts, int64_t n_expert, int64_t row_lo, int64_t row_hi, int64_t n_cols) {
+    int64_t start = 0, row_tiles = 0;
     for (int64_t e = 0; e < n_expert; ++e) {
         const int64_t end = start + counts[e];
         const int64_t lo = start < row_lo ? row_lo : start, hi = end > row_hi ? row_hi : end;
-        if (hi > lo) {
-            rows += hi - lo;
-            padded += ceil_div(hi - lo, 256) * 256;
-        }
+        if (hi > lo) row_tiles += ceil_div(hi - lo, 256);
         start = end;
     }
-    if (rows == 0) return 256;
-    const int64_t tiles = padded / 256 * ceil_div(n_cols, 256);
-    return tiles < 512 ? 128 : 256;
+    return pick_tile(row_tiles * ceil_div(n_cols, 256));
 }
 
-// Tile height for the weight-gradient product (C is [out, in] per expert): 128 when
-// 256-row tiles would be too few to occupy the chip.
-int pick_wgrad_height(int64_t n_experts_written, int64_t out_feat, int64_t in_feat) {
-    const int64_t tiles = n_experts_written * ceil_div(out_feat, 256) * ceil_div(in_feat, 256);
-    return tiles < 512 ? 128 : 256;
+// weight gradient: C is [out, in] per expert
+TileShape pick_wgrad_tile(int64_t n_experts_written, int64_t out_feat, int64_t in_feat) {
+    return pick_tile(n_experts_written * ceil_div(out_feat, 256) * ceil_div(in_feat, 256));
 }
 
 double table_flop(const SegmentTable &tab, int64_t in_feat, int64_t out_feat) {
@@ -344,12 +356,12 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
     const bool fast = is_fast(a.dtype, {a.x, a.w, a.y, a.aux, a.bias}, {a.in_feat, a.out_feat});
     FMOE_REQUIRE(a.x_row_index == nullptr || linear_forward_can_gather(a),
                  "linear_forward: rows cannot be gathered in the loader for this shape");
-    const int block_m = pick_rows_height(counts, n_expert, row_lo, row_hi, a.out_feat);
+    const TileShape tile = pick_rows_tile(counts, n_expert, row_lo, row_hi, a.out_feat);
     for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
         const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
         GemmParams prm{};
-        prm.block_m = block_m;
-        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, block_m);
+        prm.block_m = tile.bm; prm.block_n = tile.bn;
+        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, tile.bm);
         prm.profile_class = kProfGemmFwd; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
         prm.P = a.w; prm.Q = a.x; prm.C = a.y; prm.bias = a.bias; prm.aux = a.aux;
         prm.q_row_index = a.x_row_index; prm.q_index_div = a.x_index_div; prm.q_total_rows = a.x_total_rows;
@@ -373,12 +385,12 @@ int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts, int64_
     FMOE_REQUIRE(a.gy && a.w && a.gx, "linear_dgrad: NULL tensor");
     const Plan plan = plan_rows(counts, n_expert, row_lo, row_hi);
     const bool fast = is_fast(a.dtype, {a.gy, a.w, a.gx, a.aux}, {a.in_feat, a.out_feat});
-    const int block_m = pick_rows_height(counts, n_expert, row_lo, row_hi, a.in_feat);
+    const TileShape tile = pick_rows_tile(counts, n_expert, row_lo, row_hi, a.in_feat);
     for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
         const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
         GemmParams prm{};
-        prm.block_m = block_m;
-        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, block_m);
+        prm.block_m = tile.bm; prm.block_n = tile.bn;
+        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, tile.bm);
         prm.profile_class = kProfGemmDgrad; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
         prm.P = a.w; prm.Q = a.gy; prm.C = a.gx; prm.aux = const_cast<void *>(a.aux);
         prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
@@ -399,12 +411,12 @@ int grouped_linear_wgrad(const LinearWgradArgs &a, const int64_t *counts, int64_
     FMOE_REQUIRE(a.gw && (total == 0 || (a.gy && a.x)), "linear_wgrad: NULL tensor");
     const Plan plan = plan_contraction(counts, n_expert, row_lo, row_hi, last_chunk);
     const bool fast = is_fast(a.dtype, {a.gy, a.x, a.gw}, {a.in_feat, a.out_feat});
-    const int block_m = pick_wgrad_height(plan.last - plan.first + 1, a.out_feat, a.in_feat);
+    const TileShape tile = pick_wgrad_tile(plan.last - plan.first + 1, a.out_feat, a.in_feat);
     for (int e0 = plan.first; e0 <= plan.last; e0 += kMaxGroupExperts) {
         const int e1 = std::min(plan.last, e0 + kMaxGroupExperts - 1);
         GemmParams prm{};
-        prm.block_m = block_m;
-        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, block_m);
+        prm.block_m = tile.bm; prm.block_n = tile.bn;
+        fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, tile.bm);
         prm.profile_class = kProfGemmWgrad; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
         prm.P = a.x; prm.Q = a.gy; prm.C = a.gw; prm.bias_grad = fast ? a.gb : nullptr;
         prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;

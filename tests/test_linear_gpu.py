@@ -34,9 +34,24 @@ CASES = [  # rows, experts, in, out, bias, empties
 ]
 
 
+# The MFMA kernel is built for three tile shapes (256 x 256 and 128 x 256 with eight waves, 128 x 128
+# with four); the library picks one from the launch's tile count.  FMOE_GEMM_TILE forces one, so
+# that every shape runs every case.
+TILES = [None, "256x256", "128x256", "128x128"]
+
+
+@pytest.fixture(params=TILES, ids=lambda t: t or "auto")
+def tile(request, monkeypatch):
+    if request.param is None:
+        monkeypatch.delenv("FMOE_GEMM_TILE", raising=False)
+    else:
+        monkeypatch.setenv("FMOE_GEMM_TILE", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("rows,e,fin,fout,bias,empties", CASES)
-def test_linear_forward_backward(dtype, rows, e, fin, fout, bias, empties, device):
+def test_linear_forward_backward(dtype, rows, e, fin, fout, bias, empties, device, tile):
     g = torch.Generator().manual_seed(rows + e + fin)
     counts = ragged_counts(rows, e, g, empties) if rows else torch.zeros(e, dtype=torch.int64)
     x = (torch.randn(rows, fin, generator=g)).to(dtype)
@@ -67,7 +82,7 @@ def test_linear_forward_backward(dtype, rows, e, fin, fout, bias, empties, devic
 # elements each): contraction lengths of one to five slabs, with and without a ragged tail,
 # for the forward/data-grad (contraction = features) and the weight-grad (contraction = the
 # expert's rows), several row and column tiles per expert, and both tile heights (launches
-# of 512 tiles and more use 256-row tiles, smaller ones 128).
+# of 512 tiles and more use 256-row tiles, smaller ones 128) -- and every tile shape forced.
 DEPTH_CASES = [  # rows, experts, in, out
     (300, 2, 64, 264),      # one slab (bf16), column tail
     (520, 2, 128, 256),     # two slabs
@@ -82,7 +97,7 @@ DEPTH_CASES = [  # rows, experts, in, out
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,e,fin,fout", DEPTH_CASES)
-def test_linear_pipeline_depths(dtype, rows, e, fin, fout, device):
+def test_linear_pipeline_depths(dtype, rows, e, fin, fout, device, tile):
     g = torch.Generator().manual_seed(rows * 7 + fin)
     counts = ragged_counts(rows, e, g, 0)
     x = torch.randn(rows, fin, generator=g).to(dtype)
@@ -151,15 +166,18 @@ def test_linearity_at_full_width(device):
     assert rel_err(y1[:700], ref) <= 2e-2
 
 
+@pytest.mark.parametrize("forced_tile", ["128x256", "256x256", "128x128"])
 @pytest.mark.parametrize("fin,fout", [(14336, 4096), (4096, 14336)])
-def test_full_depth_bf16_forward_backward(fin, fout, device):
+def test_full_depth_bf16_forward_backward(fin, fout, forced_tile, device, monkeypatch):
     """The Mixtral-like share's feature sizes at full contraction depth, both linears: bf16 forward,
     data-grad (contraction 4096 / 14336), weight-grad and bias-grad against the float64 oracle, on
     ragged segments that leave partial row tiles; normwise AND element by element (|d| <= tol |ref| +
-    tol rms(ref)).  Both the forward and the data-grad launch fill less than half a round of the chip
-    after their whole rounds, so they also run the contraction-split tail with its fp32 partial sums."""
+    tol rms(ref)).  With 128 x 256 tiles both the forward and the data-grad launch fill less than half
+    a round of the chip after their whole rounds, so they also run the contraction-split tail with its
+    fp32 partial sums."""
     import ctypes
     from fastermoe_amd import _lib
+    monkeypatch.setenv("FMOE_GEMM_TILE", forced_tile)
     g = torch.Generator().manual_seed(fin // 7)
     counts = torch.tensor([350, 0, 250])
     rows, e = 600, 3
@@ -167,9 +185,9 @@ def test_full_depth_bf16_forward_backward(fin, fout, device):
     w = (torch.randn(e, fout, fin, generator=g) / fin ** 0.5).bfloat16()
     b = torch.randn(e, fout, generator=g).bfloat16()
     gy = torch.randn(rows, fout, generator=g).bfloat16()
-    # 128-row tiles (fewer than 512 tiles of 256): 3 + 2 row tiles; both products are split
+    # 128-row tiles: 3 + 2 row tiles; both products are split
     plan = (ctypes.c_int64 * 3)()
-    for width, depth in ((fout, fin), (fin, fout)):
+    for width, depth in ((fout, fin), (fin, fout)) if forced_tile == "128x256" else ():
         _lib.check(_lib.load().fmoe_gemm_tail_plan(5 * ((width + 255) // 256), (depth + 63) // 64, 256,
                                                   ctypes.cast(plan, ctypes.c_void_p)))
         assert plan[1] > 1
@@ -184,9 +202,10 @@ def test_full_depth_bf16_forward_backward(fin, fout, device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_contraction_split_tail_matches_oracle(dtype, device):
-    """A launch of (2 + 1) x 20 row/column tiles whose contraction (80 slabs of bf16, 160 of fp32)
-    is split into parts: forward with bias and data-grad, with a ragged contraction tail."""
+def test_contraction_split_tail_matches_oracle(dtype, device, monkeypatch):
+    """A launch of (2 + 1) x 20 row/column tiles (128 x 256) whose contraction (80 slabs of bf16, 160
+    of fp32) is split into parts: forward with bias and data-grad, with a ragged contraction tail."""
+    monkeypatch.setenv("FMOE_GEMM_TILE", "128x256")
     g = torch.Generator().manual_seed(23)
     counts = torch.tensor([200, 100])
     fin, fout = 5120 - 8, 5120 - 24
