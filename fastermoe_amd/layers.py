@@ -161,7 +161,8 @@ class FMoE(nn.Module):
         input_ptr = 0
         for j, counts in enumerate(fwd_expert_count.view(-1, num_expert)):
             size = int(counts.sum().item())
-            node_inp = inp[input_ptr:input_ptr + size]
+            # (a slice of all rows would still put a zero-fill and a copy of [rows, d] into the backward)
+            node_inp = inp if input_ptr == 0 and size == inp.shape[0] else inp[input_ptr:input_ptr + size]
             input_ptr += size
             experts = models[j]
             if not experts:
@@ -178,7 +179,7 @@ class FMoE(nn.Module):
                 outputs.append(experts[i](node_inp[base_idx:base_idx + batch_size]))
                 base_idx += batch_size
             res.append(torch.cat(outputs, dim=0))
-        return torch.cat(res, dim=0)
+        return res[0] if len(res) == 1 else torch.cat(res, dim=0)
 
     def mark_parallel_comm(self, expert_dp_comm="none"):
         r"""fmoe/layers.py:257-270."""
