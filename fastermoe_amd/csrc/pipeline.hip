@@ -22,6 +22,7 @@
 #include "grouped_gemm.hpp"
 #include "permute.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 #include <mutex>
 #include <vector>
@@ -67,6 +68,21 @@ int get_lanes(DeviceLanes **out) {
     return FMOE_OK;
 }
 
+// The streams a call enqueues on: the library's three lanes, or -- with a single chunk, where
+// nothing can overlap -- the caller's own stream for everything, with no events at all.
+struct CallStreams {
+    hipStream_t in, compute, out;
+    bool lanes;  // false: all three are the caller's stream
+};
+inline int record(const CallStreams &cs, hipEvent_t ev, hipStream_t s) {
+    if (cs.lanes) FMOE_HIP_CHECK(hipEventRecord(ev, s));
+    return FMOE_OK;
+}
+inline int wait(const CallStreams &cs, hipStream_t s, hipEvent_t ev) {
+    if (cs.lanes) FMOE_HIP_CHECK(hipStreamWaitEvent(s, ev, 0));
+    return FMOE_OK;
+}
+
 int fork_lanes(DeviceLanes *l, hipStream_t caller) {
     FMOE_HIP_CHECK(hipEventRecord(l->fork, caller));
     FMOE_HIP_CHECK(hipStreamWaitEvent(l->in, l->fork, 0));
@@ -97,7 +113,8 @@ int check_common(const char *who, const fmoe_mlp_params *p, const int64_t *count
     FMOE_REQUIRE(n_tokens >= 0 && top_k >= 1 && n_rows >= 0 && n_rows <= n_tokens * top_k,
                  "%s: n_tokens=%lld top_k=%lld n_rows=%lld", who, (long long)n_tokens, (long long)top_k,
                  (long long)n_rows);
-    FMOE_REQUIRE(n_chunks >= 1 && n_chunks <= kMaxChunks, "%s: n_chunks=%d (1..%d)", who, n_chunks, kMaxChunks);
+    FMOE_REQUIRE(n_chunks >= 0 && n_chunks <= kMaxChunks, "%s: n_chunks=%d (0 = chosen by the library, 1..%d)", who,
+                 n_chunks, kMaxChunks);
     FMOE_REQUIRE(counts != nullptr, "%s: expert_count_host is NULL", who);
     int64_t s = 0;
     for (int64_t e = 0; e < p->n_expert; ++e) {
@@ -154,6 +171,19 @@ void chunk_bounds(const int64_t *counts, int64_t n_expert, int64_t n_rows, int n
     bounds[n_chunks] = n_rows;
 }
 
+// Chunk count when the caller leaves it to the library (n_chunks == 0): up to kAutoChunks, but
+// only as many as leave every chunk at least four rounds of tiles in its narrower product --
+// shorter launches lose more to partly filled rounds than the overlapped permutes gain (measured:
+// 16384 tokens x top-2, d 1024 / h 4096: 1 chunk 2.16 ms per step, 2 chunks 2.27, 4 chunks 2.73).
+constexpr int kAutoChunks = 4;
+int auto_chunks(const int64_t *counts, int64_t n_expert, int64_t d_model, int64_t d_hidden, int cus) {
+    int64_t tiles = 0;
+    for (int64_t e = 0; e < n_expert; ++e) tiles += ceil_div(counts[e], kTileRows);
+    const int64_t narrow = std::min(ceil_div(d_model, 256), ceil_div(d_hidden, 256));
+    const int64_t min_tiles = std::max<int64_t>(1, ceil_div((int64_t)4 * cus, narrow));
+    return (int)std::max<int64_t>(1, std::min<int64_t>(kAutoChunks, tiles / min_tiles));
+}
+
 int compute_units_or_default() {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 256; }
@@ -179,7 +209,7 @@ using namespace fmoe;
 extern "C" int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert, int n_chunks,
                                        int64_t d_model, int64_t d_hidden, int compute_units, int64_t *bounds_host) {
     FMOE_REQUIRE(expert_count_host && bounds_host && n_expert >= 1, "fmoe_fused_chunk_bounds: bad argument");
-    FMOE_REQUIRE(n_chunks >= 1 && n_chunks <= kMaxChunks, "fmoe_fused_chunk_bounds: n_chunks=%d (1..%d)", n_chunks,
+    FMOE_REQUIRE(n_chunks >= 0 && n_chunks <= kMaxChunks, "fmoe_fused_chunk_bounds: n_chunks=%d (0..%d)", n_chunks,
                  kMaxChunks);
     FMOE_REQUIRE(d_model >= 1 && d_hidden >= 1 && compute_units >= 0, "fmoe_fused_chunk_bounds: bad sizes");
     int64_t rows = 0;
@@ -187,8 +217,15 @@ extern "C" int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t
         FMOE_REQUIRE(expert_count_host[e] >= 0, "fmoe_fused_chunk_bounds: negative expert count");
         rows += expert_count_host[e];
     }
-    chunk_bounds(expert_count_host, n_expert, rows, n_chunks, d_model, d_hidden,
-                 compute_units > 0 ? compute_units : compute_units_or_default(), bounds_host);
+    const int cus = compute_units > 0 ? compute_units : compute_units_or_default();
+    if (n_chunks == 0) {
+        // the library's own choice: bounds of that many chunks, the entries up to kAutoChunks repeat the end
+        const int n = auto_chunks(expert_count_host, n_expert, d_model, d_hidden, cus);
+        chunk_bounds(expert_count_host, n_expert, rows, n, d_model, d_hidden, cus, bounds_host);
+        for (int c = n + 1; c <= kAutoChunks; ++c) bounds_host[c] = rows;
+        return FMOE_OK;
+    }
+    chunk_bounds(expert_count_host, n_expert, rows, n_chunks, d_model, d_hidden, cus, bounds_host);
     return FMOE_OK;
 }
 
@@ -217,13 +254,17 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
     DeviceLanes *l;
     if (int rc = get_lanes(&l)) return rc;
     std::lock_guard<std::mutex> enqueue_lock(g_enqueue_mutex[l - g_lanes]);
-    if (int rc = fork_lanes(l, caller)) return rc;
+    const int cus = compute_units_or_default();
+    if (n_chunks == 0) n_chunks = auto_chunks(expert_count_host, E, d, h, cus);
+    const CallStreams cs = n_chunks > 1 ? CallStreams{l->in, l->compute, l->out, true} : CallStreams{caller, caller, caller, false};
+    if (cs.lanes)
+        if (int rc = fork_lanes(l, caller)) return rc;
     int64_t bounds[kMaxChunks + 1];
-    chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, compute_units_or_default(), bounds);
+    chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, cus, bounds);
 
     // dropped slots become zero rows; independent of everything else
     if (out && n_rows < n_slots)
-        if (int rc = permute_zero_unmapped(slot_to_row, out, n_slots, d, dt, l->out)) return rc;
+        if (int rc = permute_zero_unmapped(slot_to_row, out, n_slots, d, dt, cs.out)) return rc;
 
     // The first GEMM reads the token rows through pos in its loader where it can; buf_in is then
     // neither written nor needed (the caller passes NULL).
@@ -236,29 +277,30 @@ extern "C" int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         // permute-in: buf_in[r] = inp[pos[r] / top_k]
-        if (int rc = permute_gather_rows(inp, pos + lo, top_k, at(buf_in, lo, d, dt), hi - lo, n_tokens, d, dt, l->in))
+        if (int rc = permute_gather_rows(inp, pos + lo, top_k, at(buf_in, lo, d, dt), hi - lo, n_tokens, d, dt, cs.in))
             return rc;
-        FMOE_HIP_CHECK(hipEventRecord(l->in_ready[c], l->in));
+        if (int rc = record(cs, l->in_ready[c], cs.in)) return rc;
     }
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
-        if (!in_loader) FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
+        if (!in_loader)
+            if (int rc = wait(cs, cs.compute, l->in_ready[c])) return rc;
         LinearForwardArgs f1{buf_in, p->w1, p->b1, buf_mid, buf_pre, d, h, dt, kEpiBiasAct, p->activation};
-        if (int rc = grouped_linear_forward(in_loader ? probe : f1, expert_count_host, E, lo, hi, l->compute)) return rc;
+        if (int rc = grouped_linear_forward(in_loader ? probe : f1, expert_count_host, E, lo, hi, cs.compute)) return rc;
         LinearForwardArgs f2{buf_mid, p->w2, p->b2, buf_out, nullptr, h, d, dt, kEpiStore, FMOE_ACT_NONE};
-        if (int rc = grouped_linear_forward(f2, expert_count_host, E, lo, hi, l->compute)) return rc;
-        FMOE_HIP_CHECK(hipEventRecord(l->out_ready[c], l->compute));
+        if (int rc = grouped_linear_forward(f2, expert_count_host, E, lo, hi, cs.compute)) return rc;
+        if (int rc = record(cs, l->out_ready[c], cs.compute)) return rc;
     }
     for (int c = 0; c < n_chunks && out; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
-        FMOE_HIP_CHECK(hipStreamWaitEvent(l->out, l->out_ready[c], 0));
+        if (int rc = wait(cs, cs.out, l->out_ready[c])) return rc;
         // permute-out: out[pos[r]] = buf_out[r]
-        if (int rc = permute_scatter_rows(at(buf_out, lo, d, dt), pos + lo, out, hi - lo, n_slots, d, dt, l->out))
+        if (int rc = permute_scatter_rows(at(buf_out, lo, d, dt), pos + lo, out, hi - lo, n_slots, d, dt, cs.out))
             return rc;
     }
-    return join_lanes(l, caller);
+    return cs.lanes ? join_lanes(l, caller) : FMOE_OK;
 }
 
 extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *grad_out, const int64_t *pos,
@@ -282,55 +324,59 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     DeviceLanes *l;
     if (int rc = get_lanes(&l)) return rc;
     std::lock_guard<std::mutex> enqueue_lock(g_enqueue_mutex[l - g_lanes]);
-    if (int rc = fork_lanes(l, caller)) return rc;
+    const int cus = compute_units_or_default();
+    if (n_chunks == 0) n_chunks = auto_chunks(expert_count_host, E, d, h, cus);
+    const CallStreams cs = n_chunks > 1 ? CallStreams{l->in, l->compute, l->out, true} : CallStreams{caller, caller, caller, false};
+    if (cs.lanes)
+        if (int rc = fork_lanes(l, caller)) return rc;
     int64_t bounds[kMaxChunks + 1];
-    chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, compute_units_or_default(), bounds);
+    chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, cus, bounds);
 
     // A forward that read the token rows in its loader kept no sorted copy of the input; the first
     // linear's weight gradient contracts over sorted rows, so the copy is made now (inp != NULL),
     // on the permute-in lane, long before that product runs.
     if (inp != nullptr && n_rows > 0) {
         FMOE_REQUIRE(pos != nullptr, "fmoe_fused_mlp_backward: pos is NULL");
-        if (int rc = permute_gather_rows(inp, pos, top_k, buf_in, n_rows, n_tokens, d, dt, l->in)) return rc;
+        if (int rc = permute_gather_rows(inp, pos, top_k, buf_in, n_rows, n_tokens, d, dt, cs.in)) return rc;
     }
-    FMOE_HIP_CHECK(hipEventRecord(l->regather, l->in));
+    if (int rc = record(cs, l->regather, cs.in)) return rc;
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
         // permute-in: g_out[r] = grad_out[pos[r]] (nothing to do when the caller filled g_out)
         if (grad_out)
-            if (int rc = permute_gather_rows(grad_out, pos + lo, 1, at(g_out, lo, d, dt), hi - lo, n_slots, d, dt, l->in))
+            if (int rc = permute_gather_rows(grad_out, pos + lo, 1, at(g_out, lo, d, dt), hi - lo, n_slots, d, dt, cs.in))
                 return rc;
-        FMOE_HIP_CHECK(hipEventRecord(l->in_ready[c], l->in));
+        if (int rc = record(cs, l->in_ready[c], cs.in)) return rc;
     }
     // Per chunk, only the products a later stage waits for: the two data gradients.
     const bool has_act = p->activation != FMOE_ACT_NONE;
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
-        FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->in_ready[c], 0));
+        if (int rc = wait(cs, cs.compute, l->in_ready[c])) return rc;
         // g_mid = (g_out . W2) * act'(pre);  g_in = g_mid . W1
         LinearDgradArgs d2{g_out, p->w2, g_mid, has_act ? buf_pre : nullptr, h, d, dt,
                            has_act ? kEpiDAct : kEpiStore, p->activation};
-        if (int rc = grouped_linear_dgrad(d2, expert_count_host, E, lo, hi, l->compute)) return rc;
+        if (int rc = grouped_linear_dgrad(d2, expert_count_host, E, lo, hi, cs.compute)) return rc;
         LinearDgradArgs d1{g_mid, p->w1, g_in, nullptr, d, h, dt, kEpiStore, FMOE_ACT_NONE};
-        if (int rc = grouped_linear_dgrad(d1, expert_count_host, E, lo, hi, l->compute)) return rc;
+        if (int rc = grouped_linear_dgrad(d1, expert_count_host, E, lo, hi, cs.compute)) return rc;
     }
     // grad_inp[t] = sum of the token's k expert-row gradients (rows of different chunks, so
     // this runs once, after all of them) -- on the permute-out lane, beside the weight gradients
-    FMOE_HIP_CHECK(hipEventRecord(l->out_ready[0], l->compute));
-    FMOE_HIP_CHECK(hipStreamWaitEvent(l->out, l->out_ready[0], 0));
+    if (int rc = record(cs, l->out_ready[0], cs.compute)) return rc;
+    if (int rc = wait(cs, cs.out, l->out_ready[0])) return rc;
     if (n_tokens > 0)
-        if (int rc = fmoe_reduce_slots(g_in, slot_to_row, grad_inp, n_tokens, top_k, n_rows, d, dt, l->out)) return rc;
+        if (int rc = fmoe_reduce_slots(g_in, slot_to_row, grad_inp, n_tokens, top_k, n_rows, d, dt, cs.out)) return rc;
     // The weight gradients contract over an expert's rows, all of which exist now: one launch
     // per linear over all rows, so an expert's gradient is accumulated in fp32 from start to end
     // and rounded once, whatever the chunking (experts without rows are zero-filled):
     // gW2 = g_out^T . mid, gb2 = colsum(g_out);  gW1 = g_mid^T . buf_in, gb1 = colsum(g_mid)
     // (the bias gradients come out of the weight-gradient kernel's first column tiles).
     LinearWgradArgs w2{g_out, buf_mid, grad_w2, grad_b2, h, d, dt};
-    if (int rc = grouped_linear_wgrad(w2, expert_count_host, E, 0, n_rows, true, l->compute)) return rc;
-    FMOE_HIP_CHECK(hipStreamWaitEvent(l->compute, l->regather, 0));
+    if (int rc = grouped_linear_wgrad(w2, expert_count_host, E, 0, n_rows, true, cs.compute)) return rc;
+    if (int rc = wait(cs, cs.compute, l->regather)) return rc;
     LinearWgradArgs w1{g_mid, buf_in, grad_w1, grad_b1, d, h, dt};
-    if (int rc = grouped_linear_wgrad(w1, expert_count_host, E, 0, n_rows, true, l->compute)) return rc;
-    return join_lanes(l, caller);
+    if (int rc = grouped_linear_wgrad(w1, expert_count_host, E, 0, n_rows, true, cs.compute)) return rc;
+    return cs.lanes ? join_lanes(l, caller) : FMOE_OK;
 }

@@ -555,7 +555,8 @@ def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2,
 
 def _fuse_chunks():
     import os
-    return max(1, int(os.environ.get("FMOE_FUSE_GRAN", "4")))
+    gran = os.environ.get("FMOE_FUSE_GRAN")
+    return 0 if gran is None else max(1, int(gran))  # 0: the library chooses
 
 
 def _unpack_params(params, has_bias):

@@ -34,9 +34,11 @@ def _activation_code(act):
 
 
 def fuse_chunks():
-    r"""Number of pipeline chunks; ``FMOE_FUSE_GRAN`` as in cuda/fused_compute.cu:21-28
-    (default 4)."""
-    return max(1, int(os.environ.get("FMOE_FUSE_GRAN", "4")))
+    r"""Number of pipeline chunks: ``FMOE_FUSE_GRAN`` when set (the variable of
+    cuda/fused_compute.cu:21-28, whose default there is 4); unset: 0, which lets the library take
+    up to 4 chunks but no more than leave every chunk enough tiles to fill the chip."""
+    gran = os.environ.get("FMOE_FUSE_GRAN")
+    return 0 if gran is None else max(1, int(gran))
 
 
 class _FusedExpertMLP(Function):

@@ -313,16 +313,28 @@ typedef struct fmoe_mlp_params {
  * from each expert's first row), and when the chunks are long enough all but
  * the last hold a tile count whose launches, for output widths d_model and
  * d_hidden, are whole rounds of `compute_units` workgroups (0: the current
- * device's count, 256 without a device).  Host only, no GPU work.  Plays the
- * part of the worker-group stepping of cuda/fused_compute.cuh:276-280. */
+ * device's count, 256 without a device).  n_chunks == 0 asks for the library's
+ * own choice, as in the two calls below: up to 4 chunks, but only as many as
+ * leave every chunk four rounds of tiles in its narrower product; bounds_host
+ * then has 5 entries, those beyond the chosen count repeat the end.  Host
+ * only, no GPU work.  Plays the part of the worker-group stepping of
+ * cuda/fused_compute.cuh:276-280. */
 int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert,
                             int n_chunks, int64_t d_model, int64_t d_hidden,
                             int compute_units, int64_t *bounds_host);
 
+/* 1 when fmoe_fused_mlp_forward can take buf_in = NULL for this layer and input
+ * (MFMA path: 16-byte aligned pointers, feature sizes that are multiples of 16
+ * bytes; token matrix below 2 GiB), else 0.  Host only. */
+int fmoe_fused_scatter_in_loader(const fmoe_mlp_params *p, const void *inp,
+                                 int64_t n_tokens);
+
 /* Forward of scatter -> Linear -> act -> Linear -> gather over `n_chunks`
  * contiguous chunks of the expert-sorted rows, chunk c+1's scatter and chunk
  * c-1's gather running beside chunk c's GEMMs on the library's own streams,
- * chained by events to `stream` (fork at entry, join at exit).
+ * chained by events to `stream` (fork at entry, join at exit).  n_chunks == 0:
+ * the library chooses (see fmoe_fused_chunk_bounds); with a single chunk all
+ * work is enqueued on `stream` itself and no event is used.
  *   inp        [n_tokens, d_model]
  *   pos        [n_rows] int64   flat slot of every expert-sorted row
  *   slot_to_row[n_tokens*top_k] int64 (inverse of pos, -1 = dropped)
@@ -339,12 +351,6 @@ int fmoe_fused_chunk_bounds(const int64_t *expert_count_host, int64_t n_expert,
  * Replaces fmoe_cuda_fused_forward_impl at one worker,
  * cuda/fused_compute.cuh:250-388 (fmoe_cuda.fused_forward) together with the
  * _local_scatter/_local_gather around it, fmoe/fused_functions.py:22-32. */
-/* 1 when fmoe_fused_mlp_forward can take buf_in = NULL for this layer and input
- * (MFMA path: 16-byte aligned pointers, feature sizes that are multiples of 16
- * bytes; token matrix below 2 GiB), else 0.  Host only. */
-int fmoe_fused_scatter_in_loader(const fmoe_mlp_params *p, const void *inp,
-                                 int64_t n_tokens);
-
 int fmoe_fused_mlp_forward(const fmoe_mlp_params *p, const void *inp,
                            const int64_t *pos, const int64_t *slot_to_row,
                            const int64_t *expert_count_host, int64_t n_tokens,

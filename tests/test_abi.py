@@ -208,6 +208,23 @@ def test_fused_chunk_bounds_host_logic():
     rc = lib.fmoe_fused_chunk_bounds(None, 2, 3, 64, 64, 0, None)
     assert rc == -1
 
+    # n_chunks = 0, the library's own choice: up to 4 chunks, each with at least four rounds of tiles in
+    # its narrower product (5 entries come back, those past the chosen count repeat the end)
+    def auto(counts, d, h, cus=256):
+        c = (ctypes.c_int64 * len(counts))(*counts)
+        b = (ctypes.c_int64 * 5)()
+        _lib.check(lib.fmoe_fused_chunk_bounds(ctypes.cast(c, ctypes.c_void_p), len(counts), 0, d, h, cus,
+                                               ctypes.cast(b, ctypes.c_void_p)))
+        return list(b)
+
+    assert auto(counts, 4096, 14336) == bounds(counts, 4)           # 256 row tiles x 16: 4 rounds per chunk
+    total = 16 * 2048
+    assert auto([2048] * 16, 1024, 4096) == [0] + [total] * 4       # 128 row tiles x 4 = 2 rounds: one chunk
+    two = auto([256] * 256, 2048, 1024)                             # 256 row tiles x 4 = 4 rounds: one chunk
+    assert two == [0] + [65536] * 4
+    assert auto([4096] * 32, 2048, 1024)[:3] == bounds([4096] * 32, 2, 2048, 1024)   # 512 row tiles: two chunks
+    assert auto([0, 0], 64, 64) == [0, 0, 0, 0, 0]
+
 
 def test_gemm_tail_plan_host_logic():
     """Which tiles of a launch are split along the contraction (host only)."""
