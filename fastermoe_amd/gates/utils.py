@@ -1,4 +1,6 @@
 r"""Capacity helpers of the gates (fmoe/gates/utils.py:9-26)."""
+import math
+
 import torch
 
 from .. import fmoe_native
@@ -20,3 +22,9 @@ def limit_by_capacity(topk_idx, num_expert, world_size, capacity):
         pruned = fmoe_native.prune_gate_by_capacity(topk_idx.contiguous(), new_lec.to(torch.int32),
                                                     num_expert, world_size)
     return new_lec, new_gec, pruned
+
+
+def capacity_of(rates, training, n_tokens):
+    r"""Slots an expert may take: ``rates = (train, eval)`` factors of the token count, rounded up
+    (fmoe/gates/gshard_gate.py:36-37, switch_gate.py:40-41)."""
+    return math.ceil(rates[0 if training else 1] * n_tokens)
