@@ -117,78 +117,57 @@ class FMoE(nn.Module):
         super().__init__()
         if world_size != 1:
             raise NotImplementedError("fastermoe_amd implements the single-GPU path: world_size must be 1")
-        self.num_expert = num_expert
-        self.d_model = d_model
-        self.world_size = world_size
-        self.mp_group = mp_group
-        if mp_group is None:
-            self.mp_size = 1
-            self.mp_rank = 0
-        else:
-            self.mp_size = mp_group.size()
-            self.mp_rank = mp_group.rank()
-            if self.mp_size != 1:
-                raise NotImplementedError("model-parallel groups larger than 1 are not supported")
-        self.top_k = top_k
-        if type(expert) is list:
-            self.experts = nn.ModuleList([e(d_model) for e in expert])
-            self.experts_fused = False
-            self.num_expert = num_expert = len(expert)
-        elif expert is not None:
-            self.experts = nn.ModuleList([expert(d_model) for _ in range(num_expert)])
-            self.experts_fused = False
-        else:
-            self.experts_fused = True
-        self.gate = gate(d_model, num_expert, world_size, top_k)
-        if hasattr(self.gate, "stored_models"):
-            self.gate.policy_fn = policy_fn
-        self.gate_hook = gate_hook
-        self.mask = mask
-        self.mask_dict = mask_dict
-        self.moe_group = moe_group
+        self.d_model, self.top_k, self.world_size = d_model, top_k, world_size
+        self.mp_group, self.moe_group = mp_group, moe_group
+        self.mp_size, self.mp_rank = (1, 0) if mp_group is None else (mp_group.size(), mp_group.rank())
+        if self.mp_size != 1:
+            raise NotImplementedError("model-parallel groups larger than 1 are not supported")
 
-        if os.environ.get("FMOE_ENABLE_FUSE", "0") == "1":
-            enable_fuse = True
-        self.enable_fuse = enable_fuse
-        if enable_fuse:
-            assert self.experts_fused
+        # `expert`: one module class for every expert, a list with one class per expert (its length
+        # then is the expert count), or None when the sub-class sets a fused `self.experts` itself
+        classes = expert if type(expert) is list else (None if expert is None else [expert] * num_expert)
+        self.experts_fused = classes is None
+        if classes is not None:
+            num_expert = len(classes)
+            self.experts = nn.ModuleList([cls(d_model) for cls in classes])
+        self.num_expert = num_expert
+
+        self.gate = gate(d_model, num_expert, world_size, top_k)
         self.policy_fn = policy_fn
+        if hasattr(self.gate, "stored_models"):   # gates that shadow experts take the policy too
+            self.gate.policy_fn = policy_fn
+        self.gate_hook, self.mask, self.mask_dict = gate_hook, mask, mask_dict
+
+        self.enable_fuse = enable_fuse or os.environ.get("FMOE_ENABLE_FUSE", "0") == "1"
+        if self.enable_fuse and not self.experts_fused:
+            raise AssertionError("enable_fuse needs the fused experts module of a sub-class")
 
     def expert_fn(self, inp, models, fwd_expert_count, num_expert):
-        r"""Runs the experts on expert-sorted rows (fmoe/layers.py:222-255): the
-        fused expert module in one call, or one module per row slice."""
-        res = []
-        input_ptr = 0
-        for j, counts in enumerate(fwd_expert_count.view(-1, num_expert)):
-            size = int(counts.sum().item())
-            # (a slice of all rows would still put a zero-fill and a copy of [rows, d] into the backward)
-            node_inp = inp if input_ptr == 0 and size == inp.shape[0] else inp[input_ptr:input_ptr + size]
-            input_ptr += size
-            experts = models[j]
-            if not experts:
-                if counts.any():
-                    raise ValueError(f"Experts is {experts} yet counts is {counts}")
-                continue
-            if self.experts_fused:
-                res.append(experts[0](node_inp, counts))
-                continue
-            outputs = []
-            base_idx = 0
-            for i in range(self.num_expert):
-                batch_size = int(counts[i].item())
-                outputs.append(experts[i](node_inp[base_idx:base_idx + batch_size]))
-                base_idx += batch_size
-            res.append(torch.cat(outputs, dim=0))
-        return res[0] if len(res) == 1 else torch.cat(res, dim=0)
+        r"""Runs the experts on expert-sorted rows (fmoe/layers.py:222-255): the fused expert
+        module in one call, or one module per expert on its segment of the rows.  One worker, so
+        ``fwd_expert_count`` is a single row of counts and ``models`` holds this worker's experts."""
+        counts = fwd_expert_count.view(-1, num_expert)
+        if counts.shape[0] != 1 or len(models) != 1:
+            raise NotImplementedError("expert_fn: one worker only")
+        counts, experts = counts[0], models[0]
+        sizes = [int(n) for n in counts.tolist()]
+        if sum(sizes) != inp.shape[0]:
+            raise ValueError(f"expert counts {sizes} do not add up to the {inp.shape[0]} rows given")
+        if not experts:
+            raise ValueError(f"Experts is {experts} yet counts is {counts}")
+        if self.experts_fused:
+            return experts[0](inp, counts)
+        # split (not slices): its backward is one concatenation, not a zero-filled copy per expert
+        pieces = inp.split(sizes, dim=0)
+        return torch.cat([experts[i](piece) for i, piece in enumerate(pieces)], dim=0)
 
     def mark_parallel_comm(self, expert_dp_comm="none"):
-        r"""fmoe/layers.py:257-270."""
-        if self.experts is not None:
-            if isinstance(self.experts, list):
-                for e in self.experts:
-                    mark_module_parallel_comm(e, expert_dp_comm)
-            else:
-                mark_module_parallel_comm(self.experts, expert_dp_comm)
+        r"""Tags the experts' parameters with ``expert_dp_comm`` and the gate's with "moe"
+        (fmoe/layers.py:257-270); sub-classes call it at the end of their constructor."""
+        experts = getattr(self, "experts", None)
+        if experts is not None:
+            for module in (experts if isinstance(experts, list) else [experts]):
+                mark_module_parallel_comm(module, expert_dp_comm)
         mark_module_parallel_comm(self.gate, "moe")
 
     def _mask_kernels_apply(self, inp, gate_top_k_idx, gate_score):

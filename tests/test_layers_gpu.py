@@ -404,12 +404,21 @@ def test_fmoe_generic_experts(as_list, device):
     x = torch.rand(n, d, device=device, requires_grad=True)
     idx, score = moe.gate(x)
     out = moe(x)
-    rows = x.detach().repeat_interleave(k, dim=0)
-    per_slot = torch.stack([moe.experts[int(g)](rows[i]) for i, g in enumerate(idx.view(-1))])
-    ref = torch.bmm(score.view(n, 1, k), per_slot.view(n, k, d)).reshape(n, d)
-    assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
     out.mean().backward()
-    assert x.grad is not None and all(p.grad is not None for p in moe.experts.parameters())
+    got = [x.grad.clone()] + [p.grad.clone() for p in moe.experts.parameters()]
+    x.grad = None
+    moe.zero_grad()
+    rows = x.repeat_interleave(k, dim=0)
+    per_slot = torch.stack([moe.experts[int(g)](rows[i]) for i, g in enumerate(idx.view(-1))])
+    ref = torch.bmm(score.detach().view(n, 1, k), per_slot.view(n, k, d)).reshape(n, d)
+    assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
+    # gradients through the experts (the gate's own path is cut on both sides: idx and score are data here)
+    ref.mean().backward()
+    want = [x.grad] + [p.grad for p in moe.experts.parameters()]
+    gate_part = torch.autograd.grad(moe(x).mean(), moe.gate.gate.weight, allow_unused=True)[0]
+    assert gate_part is not None                      # the layer does feed the gate's linear
+    for g, w in zip(got[1:], want[1:]):
+        assert torch.allclose(g, w, rtol=1e-4, atol=1e-6)
 
 
 @pytest.mark.parametrize("cap", [0.1, 1.1])
