@@ -38,8 +38,9 @@ CONFIGS = {
 PEAK = {"bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
 # HBM-side bytes per launch of the grouped GEMM at config 4 (rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
 # what the same counter reads for a copy kernel of known size: 1.984 and 1.000); measured offline, not in this
-# script -- the counters need their own profiler runs.
-TRAFFIC_BYTES = {"config4": {"gemm_fwd": 3.94e9, "gemm_dgrad": 3.90e9, "gemm_wgrad": 4.33e9}}
+# script -- the counters need their own profiler runs.  Per class the mean over its launches of a step: forward
+# (2.99 + 0.93 and 2.98 + 0.13 GB), data-grad (3.44 + 0.46 and 2.98 + 0.13 GB), weight-grad (16.89 + 0.94 GB, all rows).
+TRAFFIC_BYTES = {"config4": {"gemm_fwd": 3.52e9, "gemm_dgrad": 3.51e9, "gemm_wgrad": 17.8e9}}
 HBM_PEAK_GBS = 8000.0
 
 
