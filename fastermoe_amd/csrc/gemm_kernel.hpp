@@ -806,6 +806,8 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
     constexpr int NPASS = WN / CPP;
     unsigned char *stg = smem + (fixup ? 0 : wave) * (WM * kStgRow);
     const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride + n0 : nullptr;
+    const __amdgpu_buffer_rsrc_t bias_rs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(bias), 0, bias ? p_valid * (int)sizeof(T) : 0, kRsrcFlags);
     T *aux = prm.aux ? (T *)prm.aux + aux_off : nullptr;
     const bool accumulate = (RAGGED == kRaggedK) && prm.accumulate_first && ei == 0;
     constexpr int kPieceChunks = kPieceBytes / 16, kIoRows = 64 / kPieceChunks;
@@ -813,25 +815,41 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
 
     auto lds_sync = [&]() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup"); __builtin_amdgcn_wave_barrier(); };
 
+    // The tile in memory is addressed through a buffer resource at its origin (a tile's rows lie
+    // within 2 GiB of it): a row or column outside the tile gets an offset past the resource's
+    // end, which reads as zero and is dropped on a store -- no branches, so all of a pass's LDS
+    // reads (or loads) go out, kIoBatch at a time, before the first of them is waited for.
+    constexpr int kIoSteps = WM / kIoRows, kIoBatch = kIoSteps < 8 ? kIoSteps : 8;
+    static_assert(kIoSteps % kIoBatch == 0, "row groups of a wave's sub-tile come in whole batches");
+    auto tile_offset = [&](int r, int col_base) -> uint32_t {
+        return (wave_m0 + r < q_valid && col_base + io_c * CE < p_valid)
+                   ? (uint32_t)(((int64_t)(wave_m0 + r) * prm.ldc + col_base + io_c * CE) * (int64_t)sizeof(T))
+                   : kOutOfRange;
+    };
     // memory -> staging (rows/columns outside the tile read as zero)
     auto stage_in = [&](const T *src, int col_base) {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(src), 0, (int)kOutOfRange, kRsrcFlags);
 #pragma unroll
-        for (int i = 0; i < WM / kIoRows; ++i) {
-            const int r = i * kIoRows + io_r;
-            u32x4 v = u32x4{0, 0, 0, 0};
-            if (wave_m0 + r < q_valid && col_base + io_c * CE < p_valid)
-                v = *(const u32x4 *)(src + (int64_t)(wave_m0 + r) * prm.ldc + col_base + io_c * CE);
-            *(u32x4 *)(stg + r * kStgRow + io_c * 16) = v;
+        for (int i0 = 0; i0 < kIoSteps; i0 += kIoBatch) {
+            u32x4 v[kIoBatch];
+#pragma unroll
+            for (int i = 0; i < kIoBatch; ++i)
+                v[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)tile_offset((i0 + i) * kIoRows + io_r, col_base), 0, 0);
+#pragma unroll
+            for (int i = 0; i < kIoBatch; ++i) *(u32x4 *)(stg + ((i0 + i) * kIoRows + io_r) * kStgRow + io_c * 16) = v[i];
         }
     };
     // staging -> memory
     auto stage_out = [&](T *dst, int col_base) {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(dst, 0, (int)kOutOfRange, kRsrcFlags);
 #pragma unroll
-        for (int i = 0; i < WM / kIoRows; ++i) {
-            const int r = i * kIoRows + io_r;
-            const u32x4 v = *(const u32x4 *)(stg + r * kStgRow + io_c * 16);
-            if (wave_m0 + r < q_valid && col_base + io_c * CE < p_valid)
-                *(u32x4 *)(dst + (int64_t)(wave_m0 + r) * prm.ldc + col_base + io_c * CE) = v;
+        for (int i0 = 0; i0 < kIoSteps; i0 += kIoBatch) {
+            u32x4 v[kIoBatch];
+#pragma unroll
+            for (int i = 0; i < kIoBatch; ++i) v[i] = *(const u32x4 *)(stg + ((i0 + i) * kIoRows + io_r) * kStgRow + io_c * 16);
+#pragma unroll
+            for (int i = 0; i < kIoBatch; ++i)
+                __builtin_amdgcn_raw_buffer_store_b128(v[i], rs, (int)tile_offset((i0 + i) * kIoRows + io_r, col_base), 0, 0);
         }
     };
     // accumulator side: 4 consecutive columns of one row
@@ -902,11 +920,13 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
 #pragma unroll
                 for (int g = 0; g < kAccRegs / 4; ++g) {
                     const int cip = xx * MB + g * 8 + hq * 4;  // column inside this pass
-                    float b4[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (bias && col_base + cip < p_valid) {
+                    // (columns past the tile, and every column when there is no bias, read as zero)
+                    float b4[4];
+                    {
                         alignas(16) T bv[4];
-                        if (sizeof(T) == 2) *(u32x2 *)bv = *(const u32x2 *)(bias + col_base + cip);
-                        else *(u32x4 *)bv = *(const u32x4 *)(bias + col_base + cip);
+                        const int off = (col_base + cip) * (int)sizeof(T);
+                        if (sizeof(T) == 2) *(u32x2 *)bv = __builtin_amdgcn_raw_buffer_load_b64(bias_rs, off, 0, 0);
+                        else *(u32x4 *)bv = __builtin_amdgcn_raw_buffer_load_b128(bias_rs, off, 0, 0);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) b4[i] = (float)bv[i];
                     }
