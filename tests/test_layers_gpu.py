@@ -713,3 +713,71 @@ def test_scatter_in_the_gemm_loader_equals_the_scattered_copy(dtype, device, mon
     _, buf_in, _, _ = fmoe_native.fused_mlp_forward(x, pos, s2r, cnt.cpu(), ex.htoh4.weight, ex.htoh4.bias,
                                                     ex.h4toh.weight, ex.h4toh.bias, k, 2, 3)
     assert buf_in is None
+
+
+def test_mixtral_like_share_at_full_size_sampled_against_the_oracle(device, monkeypatch):
+    """The headline configuration at its full size (32768 tokens, d 4096, h 14336, 8 experts, top-2, bf16,
+    GELU, fused pipeline with 4 chunks): one forward + backward on the GPU, then
+      * output and input gradient of 48 sampled tokens against the float64 oracle run on those tokens
+        (a token's output and input gradient depend on no other token);
+      * for one expert and 8 of its hidden units, the matching rows of grad_w1 / grad_b1 and columns of
+        grad_w2, plus all of grad_b2, computed in float64 on the CPU over ALL of that expert's rows
+        (about 8000) from the textbook formulas
+            gy = score * grad_out[token],  pre_J = x W1[J]^T + b1[J],  mid_J = gelu(pre_J),
+            grad_w2[:, J] = gy^T mid_J,  g_pre_J = (gy W2[:, J]) * gelu'(pre_J),
+            grad_w1[J] = g_pre_J^T x,  grad_b1[J] = sum g_pre_J,  grad_b2 = sum gy.
+    The contraction of the weight gradients runs over the whole expert (the pipeline's chunks cut it),
+    the data gradients over 4096 / 14336, the last chunk ends in a split tail."""
+    monkeypatch.setenv("FMOE_FUSE_GRAN", "4")
+    monkeypatch.delenv("FMOE_GEMM_TILE", raising=False)
+    torch.manual_seed(4)
+    n, d, h, e, k = 32768, 4096, 14336, 8, 2
+    with torch.device(device):
+        moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+        with torch.no_grad():
+            moe.experts.htoh4.weight.mul_((d * h) ** 0.5 * d ** -0.5)   # unit-variance activations
+            moe.experts.h4toh.weight.mul_((d * h) ** 0.5 * h ** -0.5)
+            moe.experts.htoh4.bias.normal_(0, 0.1)
+            moe.experts.h4toh.bias.normal_(0, 0.1)
+        moe = moe.to(torch.bfloat16)
+        x = torch.randn(n, d).bfloat16().requires_grad_(True)
+        logits = torch.randn(n, e)
+        grad = torch.randn(n, d).bfloat16()
+    moe.enable_fuse = True
+    val, idx = torch.topk(logits, k, dim=-1)
+    score = torch.softmax(val, dim=-1).bfloat16()
+    moe.gate.forward = lambda inp: (idx, score)
+    out = moe(x)
+    out.backward(grad)
+    ex = moe.experts
+    w1, b1, w2, b2 = ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias
+
+    # -- sampled tokens: output and input gradient
+    gen = torch.Generator().manual_seed(5)
+    sample = torch.randperm(n, generator=gen)[:48].to(device)
+    ref = omoe.moe_mlp_forward_backward_per_expert(x[sample], idx[sample], score[sample], w1, b1, w2, b2, "gelu", k,
+                                                   grad_out=grad[sample], grad_dtype=torch.float32)
+    assert_close(out[sample], ref["out"], 2e-2, "output of the sampled tokens", floor=3.0)
+    assert_close(x.grad[sample], ref["grad_inp"], 2e-2, "input gradient of the sampled tokens", floor=3.0)
+    del ref
+
+    # -- one expert, 8 hidden units: weight and bias gradients over all of the expert's rows
+    f64 = torch.float64
+    e0 = 5
+    units = torch.tensor([0, 1, 255, 256, 7000, 9999, 14334, 14335], device=device)
+    slots = torch.nonzero(idx.reshape(-1) == e0).reshape(-1)
+    tok = slots // k
+    assert slots.numel() > 7000
+    xe = x.detach()[tok].to("cpu", f64)
+    gy = score.reshape(-1)[slots].to("cpu", f64).unsqueeze(1) * grad[tok].to("cpu", f64)
+    w1_j = w1[e0][units].detach().to("cpu", f64)           # [8, d]
+    w2_j = w2[e0][:, units].detach().to("cpu", f64)        # [d, 8]
+    pre = xe @ w1_j.t() + b1[e0][units].detach().to("cpu", f64)
+    cdf = 0.5 * (1.0 + torch.erf(pre / 2.0 ** 0.5))
+    mid = pre * cdf
+    dact = cdf + pre * torch.exp(-0.5 * pre * pre) / (2.0 * math.pi) ** 0.5
+    g_pre = (gy @ w2_j) * dact
+    assert_close(w2.grad[e0][:, units], gy.t() @ mid, 2e-2, "grad_w2 columns", floor=3.0)
+    assert_close(w1.grad[e0][units], g_pre.t() @ xe, 2e-2, "grad_w1 rows", floor=3.0)
+    assert_close(b1.grad[e0][units], g_pre.sum(0), 2e-2, "grad_b1 entries", floor=3.0)
+    assert_close(b2.grad[e0], gy.sum(0), 2e-2, "grad_b2", floor=3.0)
