@@ -114,6 +114,7 @@ def test_fmoe_linear_reference_grid(num_expert, top_k, dtype, device):
 @pytest.mark.parametrize("fuse", [False, True])
 @pytest.mark.parametrize("dtype,n,d,h,e,k,act", [
     (torch.float32, 512, 512, 1024, 8, 2, "gelu"),      # config 1 shape
+    (torch.float32, 4096, 512, 1024, 8, 2, "gelu"),     # config 1 at its full size (the oracle runs it whole)
     (torch.bfloat16, 512, 1024, 4096, 16, 2, "gelu"),   # config 2 shape
     (torch.bfloat16, 768, 1024, 2048, 64, 1, "gelu"),   # config 3 routing (64 experts, Zipf top-1), half width
     (torch.bfloat16, 384, 4096, 3584, 8, 2, "gelu"),    # config 4 shape (quarter hidden)
@@ -715,23 +716,32 @@ def test_scatter_in_the_gemm_loader_equals_the_scattered_copy(dtype, device, mon
     assert buf_in is None
 
 
-def test_mixtral_like_share_at_full_size_sampled_against_the_oracle(device, monkeypatch):
-    """The headline configuration at its full size (32768 tokens, d 4096, h 14336, 8 experts, top-2, bf16,
-    GELU, fused pipeline with 4 chunks): one forward + backward on the GPU, then
+FULL_SIZE = [  # name, tokens, d_model, d_hidden, experts, top_k, fused, routing
+    ("gshard-style top-2 with capacity drops", 16384, 1024, 4096, 16, 2, False, "capacity"),
+    ("skewed switch-style top-1", 16384, 2048, 8192, 64, 1, False, "zipf"),
+    ("mixtral-like share, fused pipeline with 4 chunks", 32768, 4096, 14336, 8, 2, True, "topk"),
+    ("fine-grained top-8", 8192, 2048, 1024, 256, 8, False, "biased"),
+]
+
+
+@pytest.mark.parametrize("name,n,d,h,e,k,fuse,routing", FULL_SIZE, ids=[c[0].split(",")[0].replace(" ", "-") for c in FULL_SIZE])
+def test_bf16_configurations_at_full_size_sampled_against_the_oracle(name, n, d, h, e, k, fuse, routing, device, monkeypatch):
+    """The four bf16 benchmark configurations at their FULL size: one forward + backward on the GPU, then
       * output and input gradient of 48 sampled tokens against the float64 oracle run on those tokens
         (a token's output and input gradient depend on no other token);
-      * for one expert and 8 of its hidden units, the matching rows of grad_w1 / grad_b1 and columns of
-        grad_w2, plus all of grad_b2, computed in float64 on the CPU over ALL of that expert's rows
-        (about 8000) from the textbook formulas
+      * for the expert with the most rows and 8 of its hidden units, the matching rows of grad_w1 / grad_b1
+        and columns of grad_w2, plus all of grad_b2, computed in float64 on the CPU over ALL of that expert's
+        rows from the textbook formulas
             gy = score * grad_out[token],  pre_J = x W1[J]^T + b1[J],  mid_J = gelu(pre_J),
             grad_w2[:, J] = gy^T mid_J,  g_pre_J = (gy W2[:, J]) * gelu'(pre_J),
-            grad_w1[J] = g_pre_J^T x,  grad_b1[J] = sum g_pre_J,  grad_b2 = sum gy.
-    The contraction of the weight gradients runs over the whole expert (the pipeline's chunks cut it),
-    the data gradients over 4096 / 14336, the last chunk ends in a split tail."""
+            grad_w1[J] = g_pre_J^T x,  grad_b1[J] = sum g_pre_J,  grad_b2 = sum gy;
+      * an expert without rows (the skewed routing leaves some) has zero gradients.
+    In the fused case the contraction of the weight gradients runs over the whole expert although the
+    pipeline's chunks cut it, and the last chunk ends in a split tail."""
+    from fastermoe_amd.gates.utils import limit_by_capacity
     monkeypatch.setenv("FMOE_FUSE_GRAN", "4")
     monkeypatch.delenv("FMOE_GEMM_TILE", raising=False)
-    torch.manual_seed(4)
-    n, d, h, e, k = 32768, 4096, 14336, 8, 2
+    torch.manual_seed(e)
     with torch.device(device):
         moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
         with torch.no_grad():
@@ -741,11 +751,22 @@ def test_mixtral_like_share_at_full_size_sampled_against_the_oracle(device, monk
             moe.experts.h4toh.bias.normal_(0, 0.1)
         moe = moe.to(torch.bfloat16)
         x = torch.randn(n, d).bfloat16().requires_grad_(True)
-        logits = torch.randn(n, e)
         grad = torch.randn(n, d).bfloat16()
-    moe.enable_fuse = True
-    val, idx = torch.topk(logits, k, dim=-1)
-    score = torch.softmax(val, dim=-1).bfloat16()
+        logits = torch.randn(n, e)
+        if routing == "biased":
+            logits = logits + 0.5 * torch.randn(e)
+        if routing == "capacity":
+            logits = logits + torch.linspace(-0.6, 0.6, e)   # mild imbalance, so that some experts overflow
+    moe.enable_fuse = fuse
+    if routing == "zipf":
+        idx = zipf_experts(n, e, 1.2, torch.Generator().manual_seed(7)).view(n, 1).to(device)
+        score = torch.ones(n, 1, dtype=torch.bfloat16, device=device)
+    else:
+        val, idx = torch.topk(logits, k, dim=-1)
+        score = torch.softmax(val, dim=-1).bfloat16()
+        if routing == "capacity":
+            idx = limit_by_capacity(idx, e, 1, math.ceil(1.2 * n * k / e))[2]
+            assert 0 < int((idx < 0).sum()) < n * k // 2
     moe.gate.forward = lambda inp: (idx, score)
     out = moe(x)
     out.backward(grad)
@@ -753,21 +774,20 @@ def test_mixtral_like_share_at_full_size_sampled_against_the_oracle(device, monk
     w1, b1, w2, b2 = ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias
 
     # -- sampled tokens: output and input gradient
-    gen = torch.Generator().manual_seed(5)
-    sample = torch.randperm(n, generator=gen)[:48].to(device)
+    sample = torch.randperm(n, generator=torch.Generator().manual_seed(5))[:48].to(device)
     ref = omoe.moe_mlp_forward_backward_per_expert(x[sample], idx[sample], score[sample], w1, b1, w2, b2, "gelu", k,
                                                    grad_out=grad[sample], grad_dtype=torch.float32)
-    assert_close(out[sample], ref["out"], 2e-2, "output of the sampled tokens", floor=3.0)
-    assert_close(x.grad[sample], ref["grad_inp"], 2e-2, "input gradient of the sampled tokens", floor=3.0)
+    assert_close(out[sample], ref["out"], 2e-2, f"{name}: output of the sampled tokens", floor=3.0)
+    assert_close(x.grad[sample], ref["grad_inp"], 2e-2, f"{name}: input gradient of the sampled tokens", floor=3.0)
     del ref
 
-    # -- one expert, 8 hidden units: weight and bias gradients over all of the expert's rows
+    # -- the largest expert, 8 hidden units: weight and bias gradients over all of the expert's rows
     f64 = torch.float64
-    e0 = 5
-    units = torch.tensor([0, 1, 255, 256, 7000, 9999, 14334, 14335], device=device)
+    counts = torch.bincount(idx[idx >= 0].reshape(-1), minlength=e)
+    e0 = int(counts.argmax())
+    units = torch.tensor([0, 1, 255, 256, h // 2, h // 2 + 1, h - 2, h - 1], device=device)
     slots = torch.nonzero(idx.reshape(-1) == e0).reshape(-1)
     tok = slots // k
-    assert slots.numel() > 7000
     xe = x.detach()[tok].to("cpu", f64)
     gy = score.reshape(-1)[slots].to("cpu", f64).unsqueeze(1) * grad[tok].to("cpu", f64)
     w1_j = w1[e0][units].detach().to("cpu", f64)           # [8, d]
@@ -777,7 +797,10 @@ def test_mixtral_like_share_at_full_size_sampled_against_the_oracle(device, monk
     mid = pre * cdf
     dact = cdf + pre * torch.exp(-0.5 * pre * pre) / (2.0 * math.pi) ** 0.5
     g_pre = (gy @ w2_j) * dact
-    assert_close(w2.grad[e0][:, units], gy.t() @ mid, 2e-2, "grad_w2 columns", floor=3.0)
-    assert_close(w1.grad[e0][units], g_pre.t() @ xe, 2e-2, "grad_w1 rows", floor=3.0)
-    assert_close(b1.grad[e0][units], g_pre.sum(0), 2e-2, "grad_b1 entries", floor=3.0)
-    assert_close(b2.grad[e0], gy.sum(0), 2e-2, "grad_b2", floor=3.0)
+    assert_close(w2.grad[e0][:, units], gy.t() @ mid, 2e-2, f"{name}: grad_w2 columns", floor=3.0)
+    assert_close(w1.grad[e0][units], g_pre.t() @ xe, 2e-2, f"{name}: grad_w1 rows", floor=3.0)
+    assert_close(b1.grad[e0][units], g_pre.sum(0), 2e-2, f"{name}: grad_b1 entries", floor=3.0)
+    assert_close(b2.grad[e0], gy.sum(0), 2e-2, f"{name}: grad_b2", floor=3.0)
+    for empty in torch.nonzero(counts == 0).reshape(-1).tolist()[:2]:
+        assert torch.count_nonzero(w1.grad[empty]) == 0 and torch.count_nonzero(w2.grad[empty]) == 0
+        assert torch.count_nonzero(b1.grad[empty]) == 0 and torch.count_nonzero(b2.grad[empty]) == 0
