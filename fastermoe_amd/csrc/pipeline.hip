@@ -332,14 +332,6 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
     int64_t bounds[kMaxChunks + 1];
     chunk_bounds(expert_count_host, E, n_rows, n_chunks, d, h, cus, bounds);
 
-    // A forward that read the token rows in its loader kept no sorted copy of the input; the first
-    // linear's weight gradient contracts over sorted rows, so the copy is made now (inp != NULL),
-    // on the permute-in lane, long before that product runs.
-    if (inp != nullptr && n_rows > 0) {
-        FMOE_REQUIRE(pos != nullptr, "fmoe_fused_mlp_backward: pos is NULL");
-        if (int rc = permute_gather_rows(inp, pos, top_k, buf_in, n_rows, n_tokens, d, dt, cs.in)) return rc;
-    }
-    if (int rc = record(cs, l->regather, cs.in)) return rc;
     for (int c = 0; c < n_chunks; ++c) {
         const int64_t lo = bounds[c], hi = bounds[c + 1];
         if (hi == lo) continue;
@@ -349,6 +341,15 @@ extern "C" int fmoe_fused_mlp_backward(const fmoe_mlp_params *p, const void *gra
                 return rc;
         if (int rc = record(cs, l->in_ready[c], cs.in)) return rc;
     }
+    // A forward that read the token rows in its loader kept no sorted copy of the input; the first
+    // linear's weight gradient contracts over sorted rows, so the copy is made now (inp != NULL),
+    // on the permute-in lane behind the chunks' gradient rows (which the data gradients wait for),
+    // long before that product runs.
+    if (inp != nullptr && n_rows > 0) {
+        FMOE_REQUIRE(pos != nullptr, "fmoe_fused_mlp_backward: pos is NULL");
+        if (int rc = permute_gather_rows(inp, pos, top_k, buf_in, n_rows, n_tokens, d, dt, cs.in)) return rc;
+    }
+    if (int rc = record(cs, l->regather, cs.in)) return rc;
     // Per chunk, only the products a later stage waits for: the two data gradients.
     const bool has_act = p->activation != FMOE_ACT_NONE;
     for (int c = 0; c < n_chunks; ++c) {

@@ -8,7 +8,7 @@ import torch.nn as nn
 
 from . import fmoe_native
 from .functions import (AllGather, MaskRestore, MaskSelect, MOECache, MOECombine, MOEGather, MOEGatherCombine,
-                        MOELinear, MOEScatter, Slice, _prepare_forward_ex, ensure_comm, mask_index)
+                        MOELinear, MOEScatter, Slice, _prepare_forward_ex, _single_worker, ensure_comm, mask_index)
 from .gates import NaiveGate
 
 
@@ -66,19 +66,19 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
     topk = gate.shape[1] if gate.dim() == 2 else 1
     out_batch_size = inp.shape[0] * topk
 
-    inp, models, stored_models, fwd_expert_count, fwd_batch_size = MOECache.apply(
-        inp,
-        all_expert_count.view(world_size, world_size, num_expert),
-        all_global_expert_count.view(world_size, world_size, num_expert),
-        local_expert_count.view(world_size, num_expert),
-        global_expert_count.view(world_size, num_expert),
-        fwd_expert_count, policy_fn, experts, inp.shape[0], inp.shape[1], topk, num_expert,
-        world_size, fused)
+    # MOECache (fmoe/functions.py:122-194) decides which experts to shadow on other workers; with
+    # one worker it is the identity, so its results are written down directly (the autograd node
+    # and its views would only add host time between the routing's read-back and the first GEMM)
+    _single_worker(world_size, "MOECache")
+    models = [[experts]] if fused else [experts]
+    stored_models = torch.zeros(world_size * num_expert, dtype=torch.bool)
+    fwd_batch_size = int(pos.shape[0])
 
     if combine_score is not None and slot_to_row.numel() != out_batch_size:
         raise ValueError("combine_score needs one gate index per (token, k) pair")
     if enable_fuse:
-        x = MOEForward.apply(inp, models, pos // topk, pos, local_expert_count, global_expert_count,
+        # (the fused entry point takes pos and top_k; the token index pos // topk is not materialised)
+        x = MOEForward.apply(inp, models, None, pos, local_expert_count, global_expert_count,
                              stored_models, fwd_batch_size, out_batch_size, world_size, slot_to_row,
                              combine_score is None)
         if combine_score is not None:
