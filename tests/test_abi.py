@@ -276,3 +276,40 @@ def test_reference_import_paths_resolve():
     assert LayersFMoE is fastermoe_amd.FMoE and TransformerMLP is fastermoe_amd.FMoETransformerMLP
     assert importlib.import_module("fmoe.gates.naive_gate").NaiveGate is gates.NaiveGate
     assert importlib.import_module("fmoe.layers") is layers
+
+
+def test_header_is_plain_c_and_a_c_program_links(tmp_path):
+    """The boundary is a C ABI: include/fmoe_hip.h compiles as C99 (no C++ or torch types), and a C
+    program that calls host-only entry points links against the library and runs without a GPU."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    lib_path = _lib.LIB_PATH
+    src = tmp_path / "client.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "fmoe_hip.h"
+int main(void) {
+    int64_t counts[3] = {300, 0, 724};
+    int64_t bounds[3] = {-1, -1, -1};
+    if (fmoe_abi_version() < 1) return 1;
+    if (fmoe_fused_chunk_bounds(counts, 3, 2, 64, 64, 2, bounds) != FMOE_OK) return 2;
+    if (bounds[0] != 0 || bounds[2] != 1024 || bounds[1] < 0 || bounds[1] > 1024) return 3;
+    if (fmoe_fused_chunk_bounds(0, 3, 2, 64, 64, 2, bounds) != FMOE_EINVAL) return 4;
+    if (strlen(fmoe_last_error()) == 0) return 5;
+    printf("%lld %lld %lld\n", (long long)bounds[0], (long long)bounds[1], (long long)bounds[2]);
+    return 0;
+}
+''')
+    exe = tmp_path / "client"
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    build = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", include, str(src), "-o", str(exe),
+                            lib_path, f"-Wl,-rpath,{os.path.dirname(lib_path)}", "-Wl,-rpath,/opt/rocm/lib"],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+    assert run.stdout.split()[0] == "0" and run.stdout.split()[2] == "1024"
