@@ -235,3 +235,55 @@ def test_validation_errors(device):
         fmoe_native.linear_forward(x, torch.tensor([2, 2]), w.half(), None)
     with pytest.raises(ValueError, match="features"):
         fmoe_native.linear_forward(torch.zeros(4, 6, device=device), torch.tensor([2, 2]), w, None)
+
+
+@pytest.mark.parametrize("d,h,count_list,forced_tile", [
+    (128, 256, [100, 0, 333, 79], None),          # small tiles, no split
+    (5120, 5120, [200, 100], "128x256"),          # every forward / data-grad launch ends in a split tail
+])
+def test_expert_mlp_launches_replay_from_a_hip_graph(d, h, count_list, forced_tile, device, monkeypatch):
+    """The GEMM entry points neither synchronise nor allocate nor clear memory with a memset once their split
+    workspace exists, so a launch-bound sequence (the six products of a small expert MLP) can be captured
+    into a HIP graph: three replays with new inputs, eager work and synchronisations between them, each
+    compared with the eager result of the same inputs."""
+    from fastermoe_amd import _lib as lib
+    if forced_tile:
+        monkeypatch.setenv("FMOE_GEMM_TILE", forced_tile)
+    g = torch.Generator().manual_seed(11)
+    counts = torch.tensor(count_list)
+    e, rows = len(count_list), int(counts.sum())
+    w1 = (torch.randn(e, h, d, generator=g) / d ** 0.5).bfloat16().to(device)
+    b1 = torch.randn(e, h, generator=g).bfloat16().to(device)
+    w2 = (torch.randn(e, d, h, generator=g) / h ** 0.5).bfloat16().to(device)
+    x = torch.randn(rows, d, generator=g).bfloat16().to(device)
+    gy = torch.randn(rows, d, generator=g).bfloat16().to(device)
+
+    def sequence(x, gy):
+        mid, pre = fmoe_native.linear_act_forward(x, counts, w1, b1, lib.ACT_GELU, True)
+        y = fmoe_native.linear_forward(mid, counts, w2, None)
+        g_pre = fmoe_native.linear_dact_backward(gy, counts, w2, pre, lib.ACT_GELU)
+        gw2, _ = fmoe_native.linear_weight_backward(gy, mid, counts, w2, None)
+        gx, gw1, gb1 = fmoe_native.linear_backward(g_pre, x, counts, w1, b1)
+        return y, gx, gw1, gb1, gw2
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):           # warm-up on the capture stream (its split workspace gets allocated)
+        sequence(x, gy)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    xs, gys = x.clone(), gy.clone()
+    with torch.cuda.graph(graph, stream=side):
+        captured = sequence(xs, gys)
+    for step in range(3):
+        xn = torch.randn(rows, d, generator=g).bfloat16().to(device)
+        gn = torch.randn(rows, d, generator=g).bfloat16().to(device)
+        want = sequence(xn, gn)              # eager, between the replays
+        torch.cuda.synchronize()
+        xs.copy_(xn)
+        gys.copy_(gn)
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip(captured, want):
+            assert torch.equal(got, ref), f"replay {step} differs from the eager result"
