@@ -37,6 +37,7 @@ SIGNATURES = {
     "fmoe_limit_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "fmoe_prune_gate_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp]),
     "fmoe_gather_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "fmoe_gather_rows_div": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _int, _vp]),
     "fmoe_invert_index": (_int, [_vp, _i64, _vp, _i64, _vp]),
     "fmoe_reduce_slots": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "fmoe_index_add_workspace_bytes": (_i64, [_i64, _i64]),

@@ -498,6 +498,11 @@ extern "C" int fmoe_gather_rows(const void *inp, const int64_t *index, void *out
     return permute_gather_rows(inp, index, 1, out, n_out, n_inp, row_elems, dtype, (hipStream_t)stream);
 }
 
+extern "C" int fmoe_gather_rows_div(const void *inp, const int64_t *index, int64_t index_div, void *out,
+                                    int64_t n_out, int64_t n_inp, int64_t row_elems, int dtype, void *stream) {
+    return permute_gather_rows(inp, index, index_div, out, n_out, n_inp, row_elems, dtype, (hipStream_t)stream);
+}
+
 extern "C" int fmoe_invert_index(const int64_t *pos, int64_t n_pos, int64_t *inverse, int64_t n_out,
                                  void *stream) {
     FMOE_REQUIRE(n_pos >= 0 && n_out >= 0, "fmoe_invert_index: negative size");

@@ -200,13 +200,13 @@ enum ApplyMode { kApplyAssign = 0, kApplyPrune = 1 };
 // Recomputes the per-wave histograms of this workgroup's slots, turns them into
 // per-wave starting ranks (block prefix from the scan + waves before this one)
 // and walks the slots in order.
-//   assign: pos[limit_old[e] - 1 - rank] = slot   (+ slot_to_row[slot] = that)
+//   assign: pos[limit_old[e] - 1 - rank] = slot   (+ slot_to_row[slot] = that); pos[i] = -1 for i >= limit_old[E-1]
 //   prune : out[slot] = rank < limit_old[e] ? e : -1
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void rank_apply_kernel(
     const int64_t *__restrict__ gate, const int32_t *__restrict__ block_base,
     const int32_t *__restrict__ limit_old, int64_t *__restrict__ out,
-    int64_t *__restrict__ slot_to_row, int64_t n_slots, int64_t n_out, int n_expert, int nbits) {
+    int64_t *__restrict__ slot_to_row, int64_t n_slots, int64_t n_out, int n_expert, int nbits, int fill_tail) {
     extern __shared__ int32_t lds[];  // [kWavesPerBlock][n_expert]
     const int wave = threadIdx.x / kWave;
     int32_t *mine = lds + wave * n_expert;
@@ -257,6 +257,10 @@ __global__ __launch_bounds__(kBlock) void rank_apply_kernel(
             } else if (slot_to_row && i < n_slots) {
                 slot_to_row[i] = -1;
             }
+            // the entries of `out` past the last routed slot name no slot: -1, so that a row gather over
+            // the whole buffer can be launched before the host knows how many slots were routed
+            // (fill_tail: limit_old is this library's own inclusive count prefix, so its last entry is the total)
+            if (fill_tail && i < n_slots && i < n_out && i >= (int64_t)limit_old[n_expert - 1]) out[i] = -1;
         } else {
             if (i < n_slots) out[i] = (valid && rank < limit_old[key]) ? (int64_t)key : -1;
         }
@@ -489,7 +493,7 @@ extern "C" int fmoe_assign_pos(int32_t *cum_count, const int64_t *gate, int64_t 
     FMOE_LAUNCH_CHECK();
     if (int rc = allow_lds((const void *)rank_apply_kernel<kApplyAssign>, kWavesPerBlock * E * sizeof(int32_t))) return rc;
     rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
-        gate, s.block_hist, s.limit_old, pos, nullptr, n_slots, n_pos, E, ilog2_ceil(n_expert));
+        gate, s.block_hist, s.limit_old, pos, nullptr, n_slots, n_pos, E, ilog2_ceil(n_expert), 0);
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
 }
@@ -508,7 +512,7 @@ int route_launch(const int64_t *gate, int64_t n_slots, int64_t n_expert, int64_t
     FMOE_LAUNCH_CHECK();
     if (int rc = allow_lds((const void *)rank_apply_kernel<kApplyAssign>, kWavesPerBlock * E * sizeof(int32_t))) return rc;
     rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
-        gate, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert));
+        gate, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert), 1);
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
 }
@@ -611,7 +615,7 @@ extern "C" int fmoe_prune_gate_by_capacity(const int64_t *gate_idx, int64_t *new
     FMOE_LAUNCH_CHECK();
     if (int rc = allow_lds((const void *)rank_apply_kernel<kApplyPrune>, kWavesPerBlock * E * sizeof(int32_t))) return rc;
     rank_apply_kernel<kApplyPrune><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
-        gate_idx, s.block_hist, s.limit_old, new_gate_idx, nullptr, n_slots, n_slots, E, ilog2_ceil(n_expert));
+        gate_idx, s.block_hist, s.limit_old, new_gate_idx, nullptr, n_slots, n_slots, E, ilog2_ceil(n_expert), 0);
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
 }
@@ -680,7 +684,7 @@ extern "C" int fmoe_gate_topk_route(const void *logits, int64_t n_tokens, int64_
     FMOE_LAUNCH_CHECK();
     if (int rc2 = allow_lds((const void *)rank_apply_kernel<kApplyAssign>, kWavesPerBlock * E * sizeof(int32_t))) return rc2;
     rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
-        topk_idx, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert));
+        topk_idx, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert), 1);
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
 }

@@ -195,15 +195,19 @@ def _rows(name, t):
     return _float_dtype(name, t)
 
 
-def gather_rows(inp, index, n_out=None):
-    """out[r] = inp[index[r]] (zero row where index[r] < 0)."""
+def gather_rows(inp, index, n_out=None, index_div=1):
+    """out[r] = inp[index[r] // index_div] (zero row where index[r] < 0)."""
     dt = _rows("inp", inp)
     _dev("index", index, torch.int64)
     n_out = index.numel() if n_out is None else n_out
     out = torch.empty(n_out, inp.shape[1], dtype=inp.dtype, device=inp.device)
     with torch.cuda.device(inp.device):
-        check(_lib.load().fmoe_gather_rows(_ptr(inp), _ptr(index), _ptr(out), n_out, inp.shape[0], inp.shape[1],
-                                           dt, _stream(inp)))
+        if index_div == 1:
+            check(_lib.load().fmoe_gather_rows(_ptr(inp), _ptr(index), _ptr(out), n_out, inp.shape[0], inp.shape[1],
+                                               dt, _stream(inp)))
+        else:
+            check(_lib.load().fmoe_gather_rows_div(_ptr(inp), _ptr(index), int(index_div), _ptr(out), n_out,
+                                                   inp.shape[0], inp.shape[1], dt, _stream(inp)))
     return out
 
 

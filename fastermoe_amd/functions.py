@@ -59,21 +59,77 @@ def gate_topk(logits, top_k, score_mode=0):
     return idx, (torch.softmax(val, dim=-1) if score_mode == 1 else val)
 
 
+def _route_launch(gate, num_expert):
+    """Enqueues the routing of ``gate`` (or picks up the one its :class:`GateTopK` call made) and
+    returns the device tensors ``(counts [E], pos_buf [n_slots], slot_to_row [n_slots])``; nothing
+    is read back.  ``pos_buf`` holds the routed slots first and -1 after them."""
+    with torch.no_grad():
+        cached = getattr(gate, "_fmoe_route", None)
+        if cached is not None and cached[0] == gate._version and cached[1] == num_expert:
+            return cached[2:]
+        return fmoe_native.route(gate.contiguous(), num_expert)
+
+
 def _route(gate, num_expert, world_size):
     """(pos, counts, slot_to_row): one fused routing call and ONE device-to-host
     read (the counts), instead of the histogram / cumsum / ``.item()`` /
     placement sequence of fmoe/functions.py:19-42.  An index tensor that comes
     straight from :class:`GateTopK` carries its routing with it."""
     _single_worker(world_size, "count_by_gate")
+    counts, pos_buf, slot_to_row = _route_launch(gate, num_expert)
     with torch.no_grad():
-        cached = getattr(gate, "_fmoe_route", None)
-        if cached is not None and cached[0] == gate._version and cached[1] == num_expert:
-            counts, pos_buf, slot_to_row = cached[2:]
-        else:
-            counts, pos_buf, slot_to_row = fmoe_native.route(gate.contiguous(), num_expert)
         counts_cpu = counts.cpu()
         pos = pos_buf[: int(counts_cpu.sum())]
     return pos, counts, counts_cpu, slot_to_row
+
+
+class _PendingCounts:
+    """The expert counts on their way to the host: an asynchronous copy into pinned memory that
+    starts right behind the routing kernels and is waited for as late as possible, so that work
+    which does not need the counts (the row scatter) is already enqueued when the host blocks."""
+
+    _staging = {}  # (thread, device, n_expert) -> pinned int64 buffer, reused: a wait() clones out of it
+
+    def __init__(self, counts):
+        import threading
+        key = (threading.get_ident(), counts.device.index, counts.numel())
+        buf = self._staging.get(key)
+        if buf is None:
+            buf = self._staging[key] = torch.empty(counts.numel(), dtype=torch.int64, pin_memory=True)
+        self._buf = buf
+        with torch.no_grad():
+            buf.copy_(counts, non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record()
+        self.counts_cpu = None
+
+    def wait(self):
+        if self.counts_cpu is None:
+            self._event.synchronize()
+            self.counts_cpu = self._buf.clone()
+        return self.counts_cpu
+
+
+class _ScatterRouted(Function):
+    r"""``MOEScatter`` (fmoe/functions.py:196-248) for rows routed by this package's own routing
+    call, enqueued BEFORE the expert counts are on the host: the gather runs over every entry of
+    ``pos_buf`` (the entries past the routed slots are -1 and give zero rows), then the counts are
+    waited for and the routed rows ``[:n]`` are returned.  The GPU copies rows while the host
+    blocks on the counts and prepares the experts' launches, instead of idling."""
+
+    @staticmethod
+    def forward(ctx, inp, pos_buf, slot_to_row, top_k, pending):
+        buf = fmoe_native.gather_rows(inp.contiguous(), pos_buf, index_div=top_k)
+        n_rows = int(pending.wait().sum())
+        ctx.moe_args = inp.shape[0], top_k
+        ctx.save_for_backward(slot_to_row)
+        return buf[:n_rows]
+
+    @staticmethod
+    def backward(ctx, grad_buf):
+        (slot_to_row,) = ctx.saved_tensors
+        n_tokens, top_k = ctx.moe_args
+        return fmoe_native.reduce_slots(grad_buf.contiguous(), slot_to_row, n_tokens, top_k), None, None, None, None
 
 
 def count_by_gate(gate, num_expert, world_size, require_pos=True):

@@ -8,7 +8,8 @@ import torch.nn as nn
 
 from . import fmoe_native
 from .functions import (AllGather, MaskRestore, MaskSelect, MOECache, MOECombine, MOEGather, MOEGatherCombine,
-                        MOELinear, MOEScatter, Slice, _prepare_forward_ex, _single_worker, ensure_comm, mask_index)
+                        MOELinear, MOEScatter, Slice, _PendingCounts, _ScatterRouted, _prepare_forward_ex, _route_launch,
+                        _single_worker, ensure_comm, mask_index)
 from .gates import NaiveGate
 
 
@@ -60,10 +61,26 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
     over the experts' output where it lies, and the first result is ``[N, d]``."""
     from .fused_functions import MOEForward
 
-    (pos, local_expert_count, global_expert_count, all_expert_count, all_global_expert_count,
-     fwd_expert_count), slot_to_row = _prepare_forward_ex(gate, num_expert, world_size)
-
     topk = gate.shape[1] if gate.dim() == 2 else 1
+    # Unfused path on the GPU with one gate index per (token, k) pair: the row scatter is enqueued
+    # before the host reads the expert counts (which everything after it needs), so the copy runs
+    # while the host waits for them and prepares the experts' launches.
+    early = (not enable_fuse and inp.is_cuda and gate.is_cuda and inp.dim() == 2
+             and gate.numel() == inp.shape[0] * topk and inp.shape[0] > 0)
+    scattered = None
+    if early:
+        _single_worker(world_size, "count_by_gate")
+        counts_dev, pos_buf, slot_to_row = _route_launch(gate, num_expert)
+        pending = _PendingCounts(counts_dev)
+        scattered = _ScatterRouted.apply(inp, pos_buf, slot_to_row, topk, pending)
+        counts_cpu = pending.wait()
+        pos = pos_buf[: scattered.shape[0]]
+        local_expert_count = global_expert_count = all_expert_count = all_global_expert_count = counts_cpu
+        fwd_expert_count = counts_cpu.clone()
+    else:
+        (pos, local_expert_count, global_expert_count, all_expert_count, all_global_expert_count,
+         fwd_expert_count), slot_to_row = _prepare_forward_ex(gate, num_expert, world_size)
+
     out_batch_size = inp.shape[0] * topk
 
     # MOECache (fmoe/functions.py:122-194) decides which experts to shadow on other workers; with
@@ -87,9 +104,12 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
 
     # ZeroGate hands back N*top_k indices as a 1-D tensor, so the slot count can
     # exceed the token count; the per-token reduction only applies when it does not.
-    per_token = slot_to_row if slot_to_row.numel() == inp.shape[0] * topk else None
-    x = MOEScatter.apply(inp, pos // topk, local_expert_count, global_expert_count, stored_models,
-                         fwd_batch_size, world_size, per_token, topk)
+    if scattered is not None:
+        x = scattered
+    else:
+        per_token = slot_to_row if slot_to_row.numel() == inp.shape[0] * topk else None
+        x = MOEScatter.apply(inp, pos // topk, local_expert_count, global_expert_count, stored_models,
+                             fwd_batch_size, world_size, per_token, topk)
     x = expert_fn(x, models, fwd_expert_count, num_expert)
     if combine_score is not None:
         return MOEGatherCombine.apply(x, slot_to_row, combine_score, inp.shape[0], topk), stored_models

@@ -70,7 +70,7 @@ int fmoe_assign_pos(int32_t *cum_count, const int64_t *gate, int64_t *pos,
  * with two kernels, a torch.cumsum and a host read in between):
  *   expert_count [n_expert] int64  <- histogram (overwritten, not accumulated)
  *   pos          [n_slots]  int64  <- first sum(expert_count) entries as in
- *                                     fmoe_assign_pos, the rest untouched
+ *                                     fmoe_assign_pos, the rest -1
  *   slot_to_row  [n_slots]  int64  <- inverse of pos: row of each slot in the
  *                                     expert-sorted order, -1 for dropped slots
  *                                     (may be NULL) */
@@ -148,6 +148,17 @@ int fmoe_prune_gate_by_capacity(const int64_t *gate_idx, int64_t *new_gate_idx,
 int fmoe_gather_rows(const void *inp, const int64_t *index, void *out,
                      int64_t n_out, int64_t n_inp, int64_t row_elems, int dtype,
                      void *stream);
+
+/* out[r,:] = index[r] >= 0 ? inp[index[r] / index_div,:] : 0: the local scatter
+ * of fmoe/functions.py:72-74 taken straight from the slot positions
+ * (index = pos, index_div = top_k), without materialising pos // top_k
+ * (fmoe/layers.py:133).  With the -1 entries that fmoe_route leaves past the
+ * last routed slot, it can be launched over all n_slots entries of pos before
+ * the host has read the expert counts. */
+int fmoe_gather_rows_div(const void *inp, const int64_t *index,
+                         int64_t index_div, void *out, int64_t n_out,
+                         int64_t n_inp, int64_t row_elems, int dtype,
+                         void *stream);
 
 /* inverse[0..n_out) = -1, then inverse[pos[i]] = i for i in [0, n_pos).
  * With it, the zero-fill + index_copy_ of fmoe/functions.py:77-84

@@ -32,6 +32,12 @@ def test_scatter_and_gather_copy(dtype, n, k, d, drop, device):
     # scatter = index_select
     buf = _local_scatter(xd, pos // k)
     assert torch.equal(buf.cpu(), torch.index_select(x, 0, pos_c // k))
+    # the same scatter straight from the slot positions (index // k inside the kernel), over the whole position
+    # buffer: its -1 tail gives zero rows
+    cnt, pos_buf, _ = fmoe_native.route(gate.to(device), 6)
+    full = fmoe_native.gather_rows(xd, pos_buf, index_div=k)
+    assert full.shape[0] == n * k and torch.equal(full[: pos.numel()], buf)
+    assert torch.count_nonzero(full[pos.numel():]) == 0
     # gather (copy) = zeros + index_copy_
     y = torch.randn(pos.numel(), d).to(dtype)
     ref = torch.zeros(n * k, d, dtype=dtype).index_copy_(0, pos_c, y)

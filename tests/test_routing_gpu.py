@@ -106,6 +106,12 @@ def test_route_bit_exact(n, k, e, drop, device):
     assert len(out) == 6 and all(not t.is_cuda for t in out[1:])
     assert np.array_equal(out[5].numpy(), ref_cnt)
 
+    # the whole position buffer: routed slots first, -1 for the entries dropped slots leave unused
+    cnt, pos_buf, s2r = fmoe_native.route(g, e)
+    total = int(ref_cnt.sum())
+    assert pos_buf.numel() == n * k and np.array_equal(pos_buf[:total].cpu().numpy(), ref_pos)
+    assert bool((pos_buf[total:] == -1).all())
+
 
 @pytest.mark.parametrize("n,k,e,cap", [(16384, 2, 16, 2458), (16384, 1, 64, 300), (8192, 8, 256, 100),
                                        (777, 2, 5, 0), (4096, 2, 8, 10 ** 6)])
