@@ -44,6 +44,11 @@ def _host_counts(name, t, n=None):
         raise ValueError(f"{name} must be a CPU tensor (it is read on the host)")
     if t.dtype != torch.int64:
         raise TypeError(f"{name} must have dtype torch.int64, got {t.dtype}")
+    # counts that are still on their way from the device (an asynchronous read-back started by the
+    # layer) are waited for here, at the last moment before the host reads them
+    pending = getattr(t, "_fmoe_pending", None)
+    if pending is not None:
+        pending.wait()
     t = t.contiguous().view(-1)
     if n is not None and t.numel() != n:
         raise ValueError(f"{name} has {t.numel()} entries, expected {n}")
@@ -347,6 +352,9 @@ def gather_combine_backward(grad_out, rows, slot_to_row, score, n_tokens, top_k)
 # ---- per-expert linear ----------------------------------------------------------
 
 def _check_linear(input_buf, expert_count, weight, bias):
+    """Shapes and dtypes first, the counts last: reading them may have to wait for their read-back.
+    ``input_buf`` may hold more rows than the counts add up to (a buffer sized for every slot, of
+    which the routed ones come first): the rows past the counted ones are neither read nor written."""
     dt = _rows("input_buf", input_buf)
     _dev("weight", weight, input_buf.dtype)
     if weight.dim() != 3:
@@ -354,22 +362,27 @@ def _check_linear(input_buf, expert_count, weight, bias):
     n_expert, out_feat, in_feat = weight.shape
     if input_buf.shape[1] != in_feat:
         raise ValueError(f"input_buf has {input_buf.shape[1]} features, weight expects {in_feat}")
-    cnt = _host_counts("expert_count", expert_count, n_expert)
-    total = int(cnt.sum())
-    if total != input_buf.shape[0]:
-        raise ValueError(f"expert_count sums to {total} but input_buf has {input_buf.shape[0]} rows")
     if bias is not None:
         _dev("bias", bias, input_buf.dtype)
         if tuple(bias.shape) != (n_expert, out_feat):
             raise ValueError(f"bias must be [{n_expert}, {out_feat}], got {tuple(bias.shape)}")
-    return dt, cnt, n_expert, out_feat, in_feat
+    return dt, n_expert, out_feat, in_feat
+
+
+def _linear_counts(input_buf, expert_count, n_expert):
+    cnt = _host_counts("expert_count", expert_count, n_expert)
+    total = int(cnt.sum())
+    if total > input_buf.shape[0]:
+        raise ValueError(f"expert_count sums to {total} but input_buf has {input_buf.shape[0]} rows")
+    return cnt
 
 
 def linear_forward(input_buf, expert_count, weight, bias=None):
     """Y[seg_e] = X[seg_e] @ W_e^T (+ b_e).  fmoe_cuda.linear_forward,
     cuda/parallel_linear.cu:5-49; ``expert_count`` is a CPU int64 tensor."""
-    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    dt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
     out = torch.empty(input_buf.shape[0], out_feat, dtype=input_buf.dtype, device=input_buf.device)
+    cnt = _linear_counts(input_buf, expert_count, n_expert)
     with torch.cuda.device(input_buf.device):
         check(_lib.load().fmoe_linear_forward(_ptr(input_buf), _ptr(weight), _ptr(bias), _ptr(out),
                                               ctypes.c_void_p(cnt.data_ptr()), n_expert, in_feat, out_feat, dt,
@@ -382,7 +395,8 @@ def linear_backward(grad_output_buf, input_buf, expert_count, weight, bias=None)
     cuda/parallel_linear.cu:52-94.  ``grad_bias`` is computed only when ``bias``
     is given (the reference returns an uninitialised tensor otherwise); without
     bias it is ``None``."""
-    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    dt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    cnt = _linear_counts(input_buf, expert_count, n_expert)
     _dev("grad_output_buf", grad_output_buf, input_buf.dtype)
     if tuple(grad_output_buf.shape) != (input_buf.shape[0], out_feat):
         raise ValueError(f"grad_output_buf must be [{input_buf.shape[0]}, {out_feat}]")
@@ -401,12 +415,13 @@ def linear_act_forward(input_buf, expert_count, weight, bias, activation, keep_p
     """``pre = X @ W_e^T + b_e`` per expert segment and ``y = act(pre)`` in one grouped GEMM
     (the activation runs in its epilogue).  Returns ``(y, pre)``; ``pre`` is ``None`` when
     ``keep_pre`` is false.  ``activation`` is an ``ACT_*`` code of :mod:`fastermoe_amd._lib`."""
-    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    dt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
     if activation not in (_lib.ACT_NONE, _lib.ACT_RELU, _lib.ACT_GELU):
         raise ValueError(f"unknown activation code {activation}")
     new = lambda: torch.empty(input_buf.shape[0], out_feat, dtype=input_buf.dtype, device=input_buf.device)
     y = new()
     pre = new() if keep_pre else None
+    cnt = _linear_counts(input_buf, expert_count, n_expert)
     with torch.cuda.device(input_buf.device):
         check(_lib.load().fmoe_linear_act_forward(_ptr(input_buf), _ptr(weight), _ptr(bias), _ptr(pre), _ptr(y),
                                                   ctypes.c_void_p(cnt.data_ptr()), n_expert, in_feat, out_feat, dt,
@@ -426,8 +441,8 @@ def linear_dact_backward(grad_output_buf, expert_count, weight, pre, activation)
     if grad_output_buf.shape[1] != out_feat:
         raise ValueError(f"grad_output_buf has {grad_output_buf.shape[1]} features, weight produces {out_feat}")
     cnt = _host_counts("expert_count", expert_count, n_expert)
-    if int(cnt.sum()) != grad_output_buf.shape[0]:
-        raise ValueError("expert_count does not sum to the number of rows")
+    if int(cnt.sum()) > grad_output_buf.shape[0]:
+        raise ValueError("expert_count sums to more rows than grad_output_buf has")
     if activation != _lib.ACT_NONE:
         _dev("pre", pre, grad_output_buf.dtype)
         if tuple(pre.shape) != (grad_output_buf.shape[0], in_feat):
@@ -443,7 +458,8 @@ def linear_dact_backward(grad_output_buf, expert_count, weight, pre, activation)
 
 def linear_weight_backward(grad_output_buf, input_buf, expert_count, weight, bias=None):
     """The weight (and bias) half of :func:`linear_backward`: ``[grad_weight, grad_bias]``."""
-    dt, cnt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    dt, n_expert, out_feat, in_feat = _check_linear(input_buf, expert_count, weight, bias)
+    cnt = _linear_counts(input_buf, expert_count, n_expert)
     _dev("grad_output_buf", grad_output_buf, input_buf.dtype)
     if tuple(grad_output_buf.shape) != (input_buf.shape[0], out_feat):
         raise ValueError(f"grad_output_buf must be [{input_buf.shape[0]}, {out_feat}]")

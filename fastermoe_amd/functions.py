@@ -85,10 +85,13 @@ def _route(gate, num_expert, world_size):
 
 class _PendingCounts:
     """The expert counts on their way to the host: an asynchronous copy into pinned memory that
-    starts right behind the routing kernels and is waited for as late as possible, so that work
-    which does not need the counts (the row scatter) is already enqueued when the host blocks."""
+    starts right behind the routing kernels.  ``counts_cpu`` is the CPU tensor the counts will be
+    in; it carries this object as ``_fmoe_pending``, and whoever reads its values calls
+    :meth:`wait` first (``fmoe_native`` does, just before a launch that needs them), so that all
+    host work up to that point runs while the GPU is still busy with whatever precedes the
+    routing, instead of after it."""
 
-    _staging = {}  # (thread, device, n_expert) -> pinned int64 buffer, reused: a wait() clones out of it
+    _staging = {}  # (thread, device, n_expert) -> pinned int64 buffer, reused: wait() copies out of it
 
     def __init__(self, counts):
         import threading
@@ -101,35 +104,36 @@ class _PendingCounts:
             buf.copy_(counts, non_blocking=True)
         self._event = torch.cuda.Event()
         self._event.record()
-        self.counts_cpu = None
+        self._done = False
+        self.counts_cpu = torch.empty(counts.numel(), dtype=torch.int64)
+        self.counts_cpu._fmoe_pending = self
 
     def wait(self):
-        if self.counts_cpu is None:
+        if not self._done:
             self._event.synchronize()
-            self.counts_cpu = self._buf.clone()
+            self.counts_cpu.copy_(self._buf)
+            self._done = True
         return self.counts_cpu
 
 
 class _ScatterRouted(Function):
     r"""``MOEScatter`` (fmoe/functions.py:196-248) for rows routed by this package's own routing
     call, enqueued BEFORE the expert counts are on the host: the gather runs over every entry of
-    ``pos_buf`` (the entries past the routed slots are -1 and give zero rows), then the counts are
-    waited for and the routed rows ``[:n]`` are returned.  The GPU copies rows while the host
-    blocks on the counts and prepares the experts' launches, instead of idling."""
+    ``pos_buf`` (the entries past the routed slots are -1 and give zero rows) and its result, one
+    row per slot with the routed rows first, is returned as it is -- the grouped GEMMs that follow
+    take the counts for how many of its rows to touch."""
 
     @staticmethod
-    def forward(ctx, inp, pos_buf, slot_to_row, top_k, pending):
-        buf = fmoe_native.gather_rows(inp.contiguous(), pos_buf, index_div=top_k)
-        n_rows = int(pending.wait().sum())
+    def forward(ctx, inp, pos_buf, slot_to_row, top_k):
         ctx.moe_args = inp.shape[0], top_k
         ctx.save_for_backward(slot_to_row)
-        return buf[:n_rows]
+        return fmoe_native.gather_rows(inp.contiguous(), pos_buf, index_div=top_k)
 
     @staticmethod
     def backward(ctx, grad_buf):
         (slot_to_row,) = ctx.saved_tensors
         n_tokens, top_k = ctx.moe_args
-        return fmoe_native.reduce_slots(grad_buf.contiguous(), slot_to_row, n_tokens, top_k), None, None, None, None
+        return fmoe_native.reduce_slots(grad_buf.contiguous(), slot_to_row, n_tokens, top_k), None, None, None
 
 
 def count_by_gate(gate, num_expert, world_size, require_pos=True):

@@ -71,12 +71,14 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
     if early:
         _single_worker(world_size, "count_by_gate")
         counts_dev, pos_buf, slot_to_row = _route_launch(gate, num_expert)
-        pending = _PendingCounts(counts_dev)
-        scattered = _ScatterRouted.apply(inp, pos_buf, slot_to_row, topk, pending)
-        counts_cpu = pending.wait()
-        pos = pos_buf[: scattered.shape[0]]
+        # the counts are read back asynchronously and waited for where their values are first needed
+        # (the binding of the first grouped GEMM); the sorted buffers of this path hold one row per
+        # slot, the routed rows first
+        counts_cpu = _PendingCounts(counts_dev).counts_cpu
+        scattered = _ScatterRouted.apply(inp, pos_buf, slot_to_row, topk)
+        pos = pos_buf
         local_expert_count = global_expert_count = all_expert_count = all_global_expert_count = counts_cpu
-        fwd_expert_count = counts_cpu.clone()
+        fwd_expert_count = counts_cpu
     else:
         (pos, local_expert_count, global_expert_count, all_expert_count, all_global_expert_count,
          fwd_expert_count), slot_to_row = _prepare_forward_ex(gate, num_expert, world_size)
@@ -166,20 +168,28 @@ class FMoE(nn.Module):
         r"""Runs the experts on expert-sorted rows (fmoe/layers.py:222-255): the fused expert
         module in one call, or one module per expert on its segment of the rows.  One worker, so
         ``fwd_expert_count`` is a single row of counts and ``models`` holds this worker's experts."""
-        counts = fwd_expert_count.view(-1, num_expert)
-        if counts.shape[0] != 1 or len(models) != 1:
+        if fwd_expert_count.numel() != num_expert or len(models) != 1:
             raise NotImplementedError("expert_fn: one worker only")
-        counts, experts = counts[0], models[0]
-        sizes = [int(n) for n in counts.tolist()]
-        if sum(sizes) != inp.shape[0]:
-            raise ValueError(f"expert counts {sizes} do not add up to the {inp.shape[0]} rows given")
+        experts = models[0]
         if not experts:
-            raise ValueError(f"Experts is {experts} yet counts is {counts}")
+            raise ValueError(f"Experts is {experts} yet counts is {fwd_expert_count}")
         if self.experts_fused:
-            return experts[0](inp, counts)
+            # (the counts go down unread: they may still be on their way from the device; ``inp`` may
+            # hold one row per slot, of which the routed ones, as many as the counts add up to, come first)
+            # (the very tensor object, not a view of it: the pending read-back rides on it)
+            return experts[0](inp, fwd_expert_count if fwd_expert_count.dim() == 1 else fwd_expert_count.view(-1))
+        pending = getattr(fwd_expert_count, "_fmoe_pending", None)
+        if pending is not None:
+            pending.wait()
+        sizes = [int(n) for n in fwd_expert_count.view(-1).tolist()]
+        if sum(sizes) > inp.shape[0]:
+            raise ValueError(f"expert counts {sizes} add up to more than the {inp.shape[0]} rows given")
         # split (not slices): its backward is one concatenation, not a zero-filled copy per expert
-        pieces = inp.split(sizes, dim=0)
-        return torch.cat([experts[i](piece) for i, piece in enumerate(pieces)], dim=0)
+        pieces = inp.split(sizes + [inp.shape[0] - sum(sizes)], dim=0)
+        out = [experts[i](piece) for i, piece in enumerate(pieces[:-1])]
+        if pieces[-1].shape[0]:
+            out.append(out[0].new_zeros(pieces[-1].shape[0], *out[0].shape[1:]) if out else pieces[-1])
+        return torch.cat(out, dim=0)
 
     def mark_parallel_comm(self, expert_dp_comm="none"):
         r"""Tags the experts' parameters with ``expert_dp_comm`` and the gate's with "moe"

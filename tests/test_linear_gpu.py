@@ -287,3 +287,24 @@ def test_expert_mlp_launches_replay_from_a_hip_graph(d, h, count_list, forced_ti
         torch.cuda.synchronize()
         for got, ref in zip(captured, want):
             assert torch.equal(got, ref), f"replay {step} differs from the eager result"
+
+
+def test_rows_past_the_counted_ones_are_left_alone(device):
+    """A buffer with one row per slot of which only the first sum(counts) are routed (the layer's sorted
+    buffers when slots were dropped): the linears read and write the counted rows only."""
+    g = torch.Generator().manual_seed(5)
+    counts = torch.tensor([70, 0, 130])
+    rows, pad, fin, fout = 200, 57, 64, 96
+    x = torch.randn(rows + pad, fin, generator=g).bfloat16()
+    x[rows:] = float("nan")                       # must never be read
+    w = (torch.randn(3, fout, fin, generator=g) / 8).bfloat16()
+    b = torch.randn(3, fout, generator=g).bfloat16()
+    gy = torch.randn(rows + pad, fout, generator=g).bfloat16()
+    gy[rows:] = float("nan")
+    ref_y, ref_gx, ref_gw, ref_gb = _reference(x[:rows], counts, w, b, gy[:rows])
+    xd, wd, bd, gyd = x.to(device), w.to(device), b.to(device), gy.to(device)
+    y = fmoe_native.linear_forward(xd, counts, wd, bd)
+    assert y.shape[0] == rows + pad and rel_err(y[:rows], ref_y) <= 2e-2
+    gx, gw, gb = fmoe_native.linear_backward(gyd, xd, counts, wd, bd)
+    assert rel_err(gx[:rows], ref_gx) <= 2e-2 and rel_err(gw, ref_gw) <= 2e-2 and rel_err(gb, ref_gb) <= 2e-2
+    assert torch.isfinite(gw).all() and torch.isfinite(gb).all()
