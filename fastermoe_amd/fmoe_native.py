@@ -512,18 +512,24 @@ def fused_mlp_forward(inp, pos, slot_to_row, expert_count, w1, b1, w2, b2, top_k
     _dev("slot_to_row", slot_to_row, torch.int64)
     if inp.dim() != 2 or inp.shape[1] != d_model:
         raise ValueError(f"inp must be [n_tokens, {d_model}]")
-    n_tokens, n_rows = inp.shape[0], pos.numel()
+    # ``pos`` may be the whole position buffer (one entry per slot, the routed slots first): the buffers
+    # then hold a row per slot and the counts say how many of them are used.  The counts are read last:
+    # they may still be on their way from the device.
+    n_tokens, cap = inp.shape[0], pos.numel()
     if slot_to_row.numel() != n_tokens * top_k:
         raise ValueError("slot_to_row must have n_tokens * top_k entries")
-    cnt = _host_counts("expert_count", expert_count, n_expert)
     new = lambda r, c: torch.empty(r, c, dtype=inp.dtype, device=inp.device)
     lib = _lib.load()
-    in_loader = (os.environ.get("FMOE_FOLD_SCATTER", "1") != "0" and n_rows > 0
+    in_loader = (os.environ.get("FMOE_FOLD_SCATTER", "1") != "0" and cap > 0
                  and lib.fmoe_fused_scatter_in_loader(ctypes.byref(prm), _ptr(inp), n_tokens) == 1)
-    buf_in = None if in_loader else new(n_rows, d_model)
-    buf_mid, buf_out = new(n_rows, d_hidden), new(n_rows, d_model)
-    buf_pre = new(n_rows, d_hidden) if activation == _lib.ACT_GELU else None
+    buf_in = None if in_loader else new(cap, d_model)
+    buf_mid, buf_out = new(cap, d_hidden), new(cap, d_model)
+    buf_pre = new(cap, d_hidden) if activation == _lib.ACT_GELU else None
     out = new(n_tokens * top_k, d_model) if slot_order else None
+    cnt = _host_counts("expert_count", expert_count, n_expert)
+    n_rows = int(cnt.sum())
+    if n_rows > cap:
+        raise ValueError(f"expert_count sums to {n_rows} but pos has {cap} entries")
     with torch.cuda.device(inp.device):
         check(lib.fmoe_fused_mlp_forward(
             ctypes.byref(prm), _ptr(inp), _ptr(pos), _ptr(slot_to_row), ctypes.c_void_p(cnt.data_ptr()),
@@ -542,11 +548,13 @@ def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2,
     sorted copy of the input; it is rebuilt here from ``inp`` ``[n_tokens, d]``."""
     prm, n_expert, d_model, d_hidden = _mlp_params(w1, b1, w2, b2, activation)
     _dev("grad_out", grad_out, w1.dtype)
-    n_rows = pos.numel()
-    want = (n_tokens * top_k, d_model) if slot_order else (n_rows, d_model)
+    cnt = _host_counts("expert_count", expert_count, n_expert)
+    n_rows, cap = int(cnt.sum()), pos.numel()   # pos may be the whole position buffer (see the forward)
+    if n_rows > cap:
+        raise ValueError(f"expert_count sums to {n_rows} but pos has {cap} entries")
+    want = (n_tokens * top_k, d_model) if slot_order else (cap, d_model)
     if tuple(grad_out.shape) != want:
         raise ValueError(f"grad_out must be [{want[0]}, {want[1]}]")
-    cnt = _host_counts("expert_count", expert_count, n_expert)
     pre = buf_pre if buf_pre is not None else buf_mid
     dev, dty = grad_out.device, grad_out.dtype
     new = lambda *s: torch.empty(*s, dtype=dty, device=dev)
@@ -555,9 +563,9 @@ def fused_mlp_backward(grad_out, pos, slot_to_row, expert_count, w1, b1, w2, b2,
         if inp is None:
             raise ValueError("fused_mlp_backward: neither buf_in nor inp")
         _dev("inp", inp, w1.dtype)
-        buf_in = new(n_rows, d_model)
-    g_out = new(n_rows, d_model) if slot_order else grad_out
-    g_mid, g_in = new(n_rows, d_hidden), new(n_rows, d_model)
+        buf_in = new(cap, d_model)
+    g_out = new(cap, d_model) if slot_order else grad_out
+    g_mid, g_in = new(cap, d_hidden), new(cap, d_model)
     grad_inp = new(n_tokens, d_model)
     grad_w1, grad_w2 = torch.empty_like(w1), torch.empty_like(w2)
     grad_b1 = torch.empty_like(b1) if b1 is not None else None

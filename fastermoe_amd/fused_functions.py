@@ -87,5 +87,7 @@ class MOEForward:
             slot_to_row = fmoe_native.invert_index(pos_g, out_batch_size)
         act = _activation_code(experts.activation)
         return _FusedExpertMLP.apply(inp, experts.htoh4.weight, experts.htoh4.bias, experts.h4toh.weight,
-                                     experts.h4toh.bias, pos_g, slot_to_row, global_expert_count.view(-1),
+                                     experts.h4toh.bias, pos_g, slot_to_row,
+                                     # (the very tensor object when it is flat: a pending read-back rides on it)
+                                     global_expert_count if global_expert_count.dim() == 1 else global_expert_count.view(-1),
                                      top_k, act, fuse_chunks(), slot_order)

@@ -65,17 +65,19 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
     # Unfused path on the GPU with one gate index per (token, k) pair: the row scatter is enqueued
     # before the host reads the expert counts (which everything after it needs), so the copy runs
     # while the host waits for them and prepares the experts' launches.
-    early = (not enable_fuse and inp.is_cuda and gate.is_cuda and inp.dim() == 2
-             and gate.numel() == inp.shape[0] * topk and inp.shape[0] > 0)
+    early = (inp.is_cuda and gate.is_cuda and inp.dim() == 2
+             and gate.numel() == inp.shape[0] * topk and inp.shape[0] > 0
+             and (not enable_fuse or combine_score is not None))
     scattered = None
     if early:
         _single_worker(world_size, "count_by_gate")
         counts_dev, pos_buf, slot_to_row = _route_launch(gate, num_expert)
         # the counts are read back asynchronously and waited for where their values are first needed
-        # (the binding of the first grouped GEMM); the sorted buffers of this path hold one row per
-        # slot, the routed rows first
+        # (the binding of the first grouped GEMM, or of the fused pipeline); the sorted buffers of
+        # this path hold one row per slot, the routed rows first
         counts_cpu = _PendingCounts(counts_dev).counts_cpu
-        scattered = _ScatterRouted.apply(inp, pos_buf, slot_to_row, topk)
+        if not enable_fuse:
+            scattered = _ScatterRouted.apply(inp, pos_buf, slot_to_row, topk)
         pos = pos_buf
         local_expert_count = global_expert_count = all_expert_count = all_global_expert_count = counts_cpu
         fwd_expert_count = counts_cpu
