@@ -175,14 +175,23 @@ class FMoE(nn.Module):
         experts = models[0]
         if not experts:
             raise ValueError(f"Experts is {experts} yet counts is {fwd_expert_count}")
-        if self.experts_fused:
-            # (the counts go down unread: they may still be on their way from the device; ``inp`` may
-            # hold one row per slot, of which the routed ones, as many as the counts add up to, come first)
+        if self.experts_fused and getattr(experts[0], "_fmoe_counts_via_bindings", False):
+            # this package's own expert module hands the counts to the grouped-GEMM bindings unread: they
+            # may still be on their way from the device, and ``inp`` may hold one row per slot, of which
+            # the routed ones, as many as the counts add up to, come first
             # (the very tensor object, not a view of it: the pending read-back rides on it)
             return experts[0](inp, fwd_expert_count if fwd_expert_count.dim() == 1 else fwd_expert_count.view(-1))
         pending = getattr(fwd_expert_count, "_fmoe_pending", None)
         if pending is not None:
             pending.wait()
+        if self.experts_fused:
+            # any other fused expert module gets what the reference gives it: exactly the routed rows
+            # and counts it can read
+            n_rows = int(fwd_expert_count.sum())
+            out = experts[0](inp if n_rows == inp.shape[0] else inp[:n_rows], fwd_expert_count.view(-1))
+            if n_rows == inp.shape[0]:
+                return out
+            return torch.cat([out, out.new_zeros(inp.shape[0] - n_rows, *out.shape[1:])], dim=0)
         sizes = [int(n) for n in fwd_expert_count.view(-1).tolist()]
         if sum(sizes) > inp.shape[0]:
             raise ValueError(f"expert counts {sizes} add up to more than the {inp.shape[0]} rows given")

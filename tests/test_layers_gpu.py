@@ -804,3 +804,43 @@ def test_bf16_configurations_at_full_size_sampled_against_the_oracle(name, n, d,
     for empty in torch.nonzero(counts == 0).reshape(-1).tolist()[:2]:
         assert torch.count_nonzero(w1.grad[empty]) == 0 and torch.count_nonzero(w2.grad[empty]) == 0
         assert torch.count_nonzero(b1.grad[empty]) == 0 and torch.count_nonzero(b2.grad[empty]) == 0
+
+
+class _CountReadingExperts(nn.Module):
+    """A user's fused expert module: reads the counts on the host, as the reference allows."""
+
+    def __init__(self, num_expert, d_model):
+        super().__init__()
+        self.scale = nn.Parameter(torch.arange(1.0, num_expert + 1))
+        self.seen = None
+
+    def forward(self, inp, fwd_expert_count):
+        sizes = fwd_expert_count.tolist()
+        assert sum(sizes) == inp.shape[0], "a fused expert module gets exactly the routed rows"
+        self.seen = sizes
+        return inp * torch.repeat_interleave(self.scale, torch.tensor(sizes, device=inp.device)).unsqueeze(1)
+
+
+def test_user_fused_experts_get_the_routed_rows_and_readable_counts(device):
+    """The layer defers the read-back of the expert counts only for its own expert module; a user's
+    fused module sees exactly the routed rows (dropped slots are gone) and counts it can read."""
+    torch.manual_seed(3)
+    n, d, e, k = 200, 32, 4, 2
+
+    class Layer(FMoE):
+        def __init__(self):
+            super().__init__(num_expert=e, d_model=d, top_k=k, gate=NaiveGate)
+            self.experts = _CountReadingExperts(e, d)
+
+    moe = Layer().to(device)
+    x = torch.randn(n, d, device=device, requires_grad=True)
+    idx = torch.randint(-1, e, (n, k), device=device)          # -1: dropped slots
+    score = torch.rand(n, k, device=device)
+    moe.gate.forward = lambda inp: (idx, score)
+    out = moe(x)
+    assert moe.experts.seen == torch.bincount(idx[idx >= 0].view(-1).cpu(), minlength=e).tolist()
+    scale = torch.where(idx >= 0, moe.experts.scale.detach()[idx.clamp(min=0)], torch.zeros((), device=device))
+    ref = x.detach() * (score * scale).sum(dim=1, keepdim=True)
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+    out.sum().backward()
+    assert torch.allclose(x.grad, (score * scale).sum(dim=1, keepdim=True).expand(n, d), rtol=1e-5, atol=1e-6)
