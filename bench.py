@@ -41,10 +41,11 @@ PEAK = {"bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
 # script -- the counters need their own profiler runs.  Per class the mean over its launches of a step: forward
 # (2.99 + 0.93 and 2.98 + 0.13 GB), data-grad (3.44 + 0.46 and 2.98 + 0.13 GB), weight-grad (16.89 + 0.94 GB, all rows).
 TRAFFIC_BYTES = {"config4": {"gemm_fwd": 3.52e9, "gemm_dgrad": 3.51e9, "gemm_wgrad": 17.8e9}}
+TRAFFIC_SOURCE = "profiles/grouped_gemm_bf16_config4_hbm_traffic.md (rocprofv3 --pmc runs, not this run)"
 HBM_PEAK_GBS = 8000.0
 
 
-def build_layer(cfg, device):
+def build_layer(cfg, device, gate_linear=False):
     import torch
     import fastermoe_amd as fmoe
     from fastermoe_amd.gates.base_gate import BaseGate
@@ -79,8 +80,17 @@ def build_layer(cfg, device):
                 _, _, idx = limit_by_capacity(idx, self.num_expert, 1, cfg["cap"])
             return idx, score
 
+    class LinearSoftmaxGate(fmoe.gates.NaiveGate):
+        """The real thing: ``nn.Linear(d_model, experts)`` inside the step, top-k of its logits and the
+        softmax over the selected ones as scores (NaiveGate with normalised scores)."""
+
+        def forward(self, inp):
+            idx, score = gate_topk(self.gate(inp), self.top_k, score_mode=1)
+            return idx, score
+
     layer = fmoe.FMoETransformerMLP(num_expert=e, d_model=cfg["d"], d_hidden=cfg["h"], top_k=k,
-                                    gate=SyntheticGate, activation=torch.nn.GELU())
+                                    gate=LinearSoftmaxGate if gate_linear else SyntheticGate,
+                                    activation=torch.nn.GELU())
     layer.enable_fuse = cfg["fuse"]
     layer = layer.to(dtype).to(device)
     gen2 = torch.Generator().manual_seed(7)
@@ -107,22 +117,35 @@ def gemm_algorithmic_bytes(cfg, rows, experts_used):
     return 2 * per_linear * e_bytes
 
 
+def time_steps(layer, x, grad, steps, warmup):
+    """`warmup` untimed steps, then exactly `steps` timed ones between two device synchronisations
+    (host clock), every step also bracketed by HIP events on the current stream (the fused pipeline
+    forks from and joins to it).  Returns (mean ms per step by the host clock, median and mean ms per
+    step by the events)."""
+    import torch
+    for _ in range(warmup):
+        step(layer, x, grad)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        step(layer, x, grad)
+        b.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    per = sorted(a.elapsed_time(b) for a, b in ev)
+    return elapsed / steps * 1e3, per[len(per) // 2], sum(per) / len(per)
+
+
 def measure(cfg, name, device, steps, warmup, profile_steps, permutes_alone):
     """Times `steps` forward + backward steps of the layer of `cfg` (after `warmup`), then `profile_steps`
     more with the library's per-launch HIP-event brackets switched on."""
     import torch
     from fastermoe_amd import _lib, fmoe_native
     layer, x, grad = build_layer(cfg, device)
-    for _ in range(warmup):
-        step(layer, x, grad)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step(layer, x, grad)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / steps * 1e3
-    tokens_per_s = cfg["n"] * steps / elapsed
+    ms_per_step, ms_median, ms_event_mean = time_steps(layer, x, grad, steps, warmup)
+    tokens_per_s = cfg["n"] / (ms_per_step * 1e-3)
 
     # per-kernel timing: HIP events recorded by the library on the stream each kernel runs on
     _lib.profile_enable(True)
@@ -132,11 +155,24 @@ def measure(cfg, name, device, steps, warmup, profile_steps, permutes_alone):
     prof = _lib.profile_collect()
     _lib.profile_enable(False)
 
+    # rows that were routed (the layer itself never reads this number on the host)
+    n, k, d = cfg["n"], cfg["k"], cfg["d"]
+    with torch.no_grad():
+        idx, _ = layer.gate(x)
+        cnt, pos_buf, s2r = fmoe_native.route(idx.contiguous(), cfg["e"])
+        cnt_cpu = cnt.cpu()
+        rows, used = int(cnt_cpu.sum()), int((cnt_cpu > 0).sum())
+    # flop per step of every GEMM class: two products of 2 * rows * d * h each (forward: both linears; data
+    # gradient: both; weight gradient: both) -- 12 * rows * d * h per step in all
+    class_flop = 4.0 * rows * cfg["d"] * cfg["h"]
+
     kernels = {}
     for kname, (launches, ms, work) in prof.items():
         if launches == 0:
             continue
         is_gemm = kname.startswith("gemm")
+        if is_gemm:
+            work = class_flop * profile_steps
         rate = work / (ms * 1e-3) / (1e12 if is_gemm else 1e9)
         kernels[kname] = {"launches_per_step": launches / profile_steps,
                           "avg_ms": round(ms / launches, 4), "ms_per_step": round(ms / profile_steps, 4),
@@ -147,12 +183,6 @@ def measure(cfg, name, device, steps, warmup, profile_steps, permutes_alone):
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_names)
     gemm_flop = sum(kernels[k]["work_per_launch"] * kernels[k]["launches_per_step"] for k in gemm_names)
 
-    n, k, d = cfg["n"], cfg["k"], cfg["d"]
-    with torch.no_grad():
-        idx, _ = layer.gate(x)
-        cnt, pos_buf, s2r = fmoe_native.route(idx.contiguous(), cfg["e"])
-        cnt_cpu = cnt.cpu()
-        rows, used = int(cnt_cpu.sum()), int((cnt_cpu > 0).sum())
     gemm_bytes = gemm_algorithmic_bytes(cfg, rows, used)
     mfma_frac = gemm_flop / (gemm_ms * 1e-3) / 1e12 / peak
     hbm_frac = gemm_bytes / (gemm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
@@ -183,6 +213,8 @@ def measure(cfg, name, device, steps, warmup, profile_steps, permutes_alone):
                     "unit": "GB/s", "frac": round(dom_frac_hbm, 4), "bytes_per_launch": dom_bytes_per_launch,
                     "avg_launch_ms": dk["avg_ms"], "frac_of_mfma_peak": round(dom_frac_mfma, 4)}
     roofline["traffic"] = TRAFFIC_BYTES.get(name, {}).get(dominant) if cfg["fuse"] else None
+    if roofline["traffic"] is not None:
+        roofline["traffic_source"] = TRAFFIC_SOURCE
 
     permute_alone = None
     if permutes_alone:
@@ -209,7 +241,9 @@ def measure(cfg, name, device, steps, warmup, profile_steps, permutes_alone):
         del buf
     del layer, x, grad
     torch.cuda.empty_cache()
-    return {"ms_per_step": round(ms_per_step, 3), "tokens_per_s": round(tokens_per_s, 1), "kernels": kernels,
+    return {"ms_per_step": round(ms_per_step, 3), "ms_per_step_median": round(ms_median, 3),
+            "ms_per_step_event_mean": round(ms_event_mean, 3), "routed_rows": rows,
+            "tokens_per_s": round(tokens_per_s, 1), "kernels": kernels,
             "gemm_all": gemm_all, "roofline": roofline, "permute_alone": permute_alone}
 
 
@@ -223,6 +257,8 @@ def main():
     ap.add_argument("--no-other-configs", dest="other_configs", action="store_false",
                     help="skip the short runs of configurations 1, 2, 3 and 5 that follow the headline workload")
     ap.add_argument("--profile-steps", type=int, default=3)
+    ap.add_argument("--no-gate-linear", dest="gate_linear", action="store_false",
+                    help="skip the second figure with the gate's linear layer inside the step")
     ap.add_argument("--fuse", choices=["auto", "on", "off"], default="auto",
                     help="override the configuration's choice of the fused pipeline")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -295,13 +331,16 @@ def main():
     result = {
         "metric": "moe_mlp_fwd_bwd_tokens_per_s", "value": m["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": m["ms_per_step"],
+        "ms_per_step_median_hip_events": m["ms_per_step_median"], "ms_per_step_mean_hip_events": m["ms_per_step_event_mean"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"],
         "data": "synthetic",
         "config": {"workload": cfg["text"], "tokens": cfg["n"], "d_model": cfg["d"], "d_hidden": cfg["h"],
                    "experts": cfg["e"], "top_k": cfg["k"], "fused": cfg["fuse"],
                    "chunks": (int(os.environ["FMOE_FUSE_GRAN"]) if "FMOE_FUSE_GRAN" in os.environ else "chosen by the library")
                    if cfg["fuse"] else 1,
-                   "gate": "top-k over fixed seeded logits; the gate's own linear layer is not part of the step"},
+                   "routed_rows": m["routed_rows"],
+                   "gate": "top-k over fixed seeded logits; the gate's own linear layer is not part of the step "
+                           "(with_gate_linear: the same layer with nn.Linear(d_model, experts) inside the step)"},
         "roofline": m["roofline"],
         "gemm_all": m["gemm_all"],
         "kernels": m["kernels"],
@@ -309,13 +348,24 @@ def main():
         "hbm_peak_gbs": HBM_PEAK_GBS,
     }
 
+    if args.gate_linear:
+        # the same workload with the gate's own linear layer inside the step
+        layer, x, grad = build_layer(cfg, device, gate_linear=True)
+        ms, med, _ = time_steps(layer, x, grad, max(5, args.steps // 2), 3)
+        result["with_gate_linear"] = {"ms_per_step": round(ms, 3), "ms_per_step_median_hip_events": round(med, 3),
+                                      "tokens_per_s": round(cfg["n"] / (ms * 1e-3), 1),
+                                      "gate": "nn.Linear(d_model, experts) + top-k + softmax over the selected logits"}
+        del layer, x, grad
+        torch.cuda.empty_cache()
+
     if args.other_configs and args.config == "config4":
         # the other workloads (parity-test configurations), 5 warm-up + 20 timed steps each
         others = {}
         for name in ("config1", "config2", "config3", "config5"):
             o = measure(dict(CONFIGS[name]), name, device, 20, 5, 3, permutes_alone=False)
             others[name] = {"workload": CONFIGS[name]["text"], "dtype": CONFIGS[name]["dtype"],
-                            "ms_per_step": o["ms_per_step"], "tokens_per_s": o["tokens_per_s"],
+                            "ms_per_step": o["ms_per_step"], "ms_per_step_median_hip_events": o["ms_per_step_median"],
+                            "routed_rows": o["routed_rows"], "tokens_per_s": o["tokens_per_s"],
                             "gemm_ms_per_step": o["gemm_all"]["ms_per_step"],
                             "gemm_frac_of_mfma_peak": o["gemm_all"]["frac_of_mfma_peak"],
                             "gemm_frac_of_hbm_peak": o["gemm_all"]["frac_of_hbm_peak"],
@@ -325,13 +375,16 @@ def main():
 
     if not args.no_cpu_baseline:
         from oracle import moe as omoe
-        sample = {"config1": cfg["n"], "config4": 8192}.get(args.config, 4096)
+        sample = {"config1": cfg["n"], "config4": 4096}.get(args.config, 4096)
         sample = min(sample, cfg["n"])
-        tps, cores, secs = omoe.time_cpu_baseline(sample, cfg["d"], cfg["h"], cfg["e"], cfg["k"], "gelu",
-                                                  seed=1, repeats=1, threads=min(os.cpu_count() or 1, 16))
+        tps, cores, best, median = omoe.time_cpu_baseline(sample, cfg["d"], cfg["h"], cfg["e"], cfg["k"], "gelu",
+                                                          seed=1, repeats=3, threads=min(os.cpu_count() or 1, 16),
+                                                          warmup=1, return_median=True)
         result["cpu_baseline"] = {"value": round(tps, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+                                  "median_value": round(sample / median, 1),
                                   "sample": f"{sample} of {cfg['n']} tokens, same d_model/d_hidden/experts/top_k, "
-                                            f"fp32, 1 iteration fwd+bwd, {secs:.1f} s"}
+                                            f"fp32, fwd+bwd, 1 warm-up + 3 timed iterations, best {best:.1f} s, "
+                                            f"median {median:.1f} s (value = best)"}
     print(json.dumps(result))
 
 

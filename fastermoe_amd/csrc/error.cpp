@@ -8,4 +8,4 @@ char *error_buffer() {
 }  // namespace fmoe
 
 extern "C" const char *fmoe_last_error(void) { return fmoe::error_buffer(); }
-extern "C" int fmoe_abi_version(void) { return 2; }
+extern "C" int fmoe_abi_version(void) { return 3; }

@@ -6,6 +6,7 @@
 #include "profile.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -192,6 +193,11 @@ struct GemmParams {
     // the epilogue.  k_split == 1: main_tiles == total_tiles.
     float *split_ws;
     int32_t main_tiles, k_split, split_slabs, fixup;
+    // Segments from a table in device memory (segtab layout) instead of `tab`: the launch is sized
+    // for the most tiles the table can describe, the kernel reads the real counts.  tab.n is then
+    // the expert count (any number), tab.first_expert 0, and nothing is split.
+    const int32_t *dev_tab;
+    int64_t dev_rows_cap;      // host only: rows the device table was laid out for
     int32_t block_m, block_n;  // host only: tile height the segment table was built for (256 or 128) and tile width
     int32_t profile_class;     // host only: ProfileClass of this launch
     double profile_work;       // host only: flop of this launch
@@ -238,25 +244,37 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
     int split_part = -1;   // >= 0: this workgroup computes that part of the contraction of a tail tile
     int tail_index = 0;    // index of a tail tile among the tail tiles
     const bool fixup = RAGGED == kRaggedRows && prm.fixup != 0;
+    // the device table is read-only while the kernel runs and addressed uniformly: scalar loads
+    typedef const int32_t __attribute__((address_space(4))) *DevTab;
+    const DevTab dtab = (DevTab)(uintptr_t)prm.dev_tab;
+    const bool dev = prm.dev_tab != nullptr;
+    int seg_lo, seg_hi;
     {
         int tm_total, rem;
         if (RAGGED == kRaggedRows) {
             int L;
-            const int main_grid = (prm.main_tiles + 7) & ~7;
+            int main_tiles = prm.main_tiles, total_tiles = prm.total_tiles;
+            if (dev) {
+                tm_total = dtab[BM == 256 ? segtab::kTiles256 : segtab::kTiles128];
+                main_tiles = total_tiles = tm_total * prm.tiles_n;
+            } else {
+                tm_total = prm.tab.tile[prm.tab.n];
+            }
+            const int main_grid = (main_tiles + 7) & ~7;
             if (fixup) {
                 tail_index = blockIdx.x / kWaves;  // one one-wave workgroup per wave of a tail tile
-                L = prm.main_tiles + tail_index;
+                L = main_tiles + tail_index;
             } else if ((int)blockIdx.x < main_grid) {
                 const int per_xcd = main_grid >> 3;
                 L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-                if (L >= prm.main_tiles) return;
+                if (L >= main_tiles) return;
             } else {
-                const int u = blockIdx.x - main_grid, n_tail = prm.total_tiles - prm.main_tiles;
+                if (dev) return;  // the launch was sized for an upper bound of tiles
+                const int u = blockIdx.x - main_grid, n_tail = total_tiles - main_tiles;
                 split_part = u / n_tail;
                 tail_index = u - split_part * n_tail;
-                L = prm.main_tiles + tail_index;
+                L = main_tiles + tail_index;
             }
-            tm_total = prm.tab.tile[prm.tab.n];
             rem = L;
             ei = 0;
         } else {
@@ -276,16 +294,30 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
         mt = first_m + in_grp % gsz;
         nt = in_grp / gsz;
         if (RAGGED == kRaggedRows) {
-            int lo = 0, hi = prm.tab.n;  // tile[lo] <= mt < tile[hi]
-            while (hi - lo > 1) {
-                const int mid = (lo + hi) >> 1;
-                if (prm.tab.tile[mid] <= mt) lo = mid; else hi = mid;
+            if (dev) {
+                // {expert, first row, rows} of row tile mt
+                const int at = dtab[BM == 256 ? segtab::kMap256 : segtab::kMap128] + 4 * mt;
+                ei = dtab[at];
+                seg_lo = dtab[at + 1];
+                seg_hi = seg_lo + dtab[at + 2];
+            } else {
+                int lo = 0, hi = prm.tab.n;  // tile[lo] <= mt < tile[hi]
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (prm.tab.tile[mid] <= mt) lo = mid; else hi = mid;
+                }
+                ei = lo;
             }
-            ei = lo;
         }
     }
     const int expert = prm.tab.first_expert + ei;
-    const int seg_lo = prm.tab.seg[ei], seg_hi = prm.tab.seg[ei + 1];
+    if (RAGGED == kRaggedK && dev) {
+        seg_lo = dtab[segtab::kHeader + ei];
+        seg_hi = dtab[segtab::kHeader + ei + 1];
+    } else if (!(RAGGED == kRaggedRows && dev)) {
+        seg_lo = prm.tab.seg[ei];
+        seg_hi = prm.tab.seg[ei + 1];
+    }
     const int n0 = nt * BN;
 
     const T *Pb;
@@ -297,7 +329,8 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
     int64_t q_gather_bytes = 0;  // extent of the gathered matrix past this part's first contraction element
     int64_t aux_off;  // offset of this tile's origin inside C (and aux)
     if (RAGGED == kRaggedRows) {
-        const int row0 = seg_lo + (mt - prm.tab.tile[ei]) * BM;
+        // (device table: seg_lo .. seg_hi are the rows of this very tile)
+        const int row0 = dev ? seg_lo : seg_lo + (mt - prm.tab.tile[ei]) * BM;
         q_row0 = row0;
         q_valid = min(BM, seg_hi - row0);
         K = prm.k_extent;
@@ -1063,16 +1096,18 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
     constexpr int smem_epi = kWavesM * kWavesN * smem_wave_epi;
     constexpr int smem = smem_loop > smem_epi ? smem_loop : smem_epi;
     // the opt-in to more than 64 KiB of dynamic LDS is per device (and per kernel instantiation)
-    static std::once_flag configured[16];
+    // (0: not tried yet, 1: done, 2: failed -- a failure is reported by every later launch too)
+    static std::atomic<int> configured[16];
     auto kern = grouped_gemm_kernel<T, BM, BN, PS, QS, RG, EPI>;
     int dev = 0;
     FMOE_HIP_CHECK(hipGetDevice(&dev));
     FMOE_REQUIRE(dev >= 0 && dev < 16, "device index %d out of range", dev);
-    hipError_t attr_err = hipSuccess;
-    std::call_once(configured[dev], [&]() {
-        attr_err = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    });
-    FMOE_HIP_CHECK(attr_err);
+    if (configured[dev].load(std::memory_order_acquire) != 1) {
+        // (two threads may both make the call; it is idempotent)
+        const hipError_t attr_err = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        configured[dev].store(attr_err == hipSuccess ? 1 : 2, std::memory_order_release);
+        FMOE_HIP_CHECK(attr_err);
+    }
     if (prm.total_tiles <= 0) return FMOE_OK;
     prm.main_tiles = prm.total_tiles;
     prm.k_split = 1;
@@ -1084,8 +1119,10 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
         constexpr int BKE = kSlabBytes / (int)sizeof(T);
         const int n_slabs = (prm.k_extent + BKE - 1) / BKE;
         // (two 128 x 128 workgroups share a compute unit: their launches are not split)
-        const TailSplit ts = BN == 256 ? plan_tail_split(prm.total_tiles, n_slabs, device_compute_units())
-                                       : TailSplit{prm.total_tiles, 1, n_slabs};
+        // (nor is a launch over a device table, whose tile count the host does not know)
+        const TailSplit ts = (BN == 256 && prm.dev_tab == nullptr)
+                                 ? plan_tail_split(prm.total_tiles, n_slabs, device_compute_units())
+                                 : TailSplit{prm.total_tiles, 1, n_slabs};
         if (ts.k_split > 1) {
             const int tail = prm.total_tiles - ts.main_tiles;
             float *ws = split_workspace(stream, (size_t)tail * ts.k_split * BM * BN * sizeof(float));
@@ -1132,7 +1169,8 @@ int launch_for_height(GemmParams &prm, int epi, hipStream_t stream) {
     int64_t total;
     if (RG == kRaggedRows) {
         prm.tiles_m = 0;
-        total = (int64_t)prm.tab.tile[prm.tab.n] * prm.tiles_n;
+        // device table: the most row tiles its rows can make (the kernel drops the surplus workgroups)
+        total = (prm.dev_tab ? segtab::cap_tiles(prm.dev_rows_cap, prm.tab.n, BM) : (int64_t)prm.tab.tile[prm.tab.n]) * prm.tiles_n;
     } else {
         prm.tiles_m = (int)ceil_div(prm.n_rows, BM);
         total = (int64_t)prm.tab.n * prm.tiles_m * prm.tiles_n;

@@ -157,6 +157,13 @@ TileShape pick_rows_tile(const int64_t *counts, int64_t n_expert, int64_t row_lo
     return pick_tile(row_tiles * ceil_div(n_cols, 256));
 }
 
+// ragged rows over a device table: the host does not know the counts; rows_cap rows spread over
+// the experts make about rows_cap / 256 whole tiles plus a partial one for every other expert
+TileShape pick_rows_tile_estimate(int64_t rows_cap, int64_t n_expert, int64_t n_cols) {
+    const int64_t whole = rows_cap / 256;
+    return pick_tile((whole + std::min<int64_t>(n_expert, std::max<int64_t>(whole, 1)) / 2) * ceil_div(n_cols, 256));
+}
+
 // weight gradient: C is [out, in] per expert
 TileShape pick_wgrad_tile(int64_t n_experts_written, int64_t out_feat, int64_t in_feat) {
     return pick_tile(n_experts_written * ceil_div(out_feat, 256) * ceil_div(in_feat, 256));
@@ -344,8 +351,45 @@ bool linear_forward_can_gather(const LinearForwardArgs &a) {
     return a.x_total_rows >= 0 && a.x_total_rows * a.in_feat * (int64_t)dtype_bytes(a.dtype) < ((int64_t)1 << 31);
 }
 
+// checks shared by the launches over a device table; fills the parts of prm that say so
+int device_table_launch(const char *who, GemmParams &prm, const int32_t *dev_tab, int64_t rows_cap, int64_t n_expert,
+                        bool fast) {
+    FMOE_REQUIRE(fast, "%s: a launch over a device segment table needs 16-byte aligned tensors, feature sizes that are "
+                       "multiples of 16 bytes and a 16- or 32-bit float type", who);
+    FMOE_REQUIRE(n_expert >= 1 && n_expert <= (int64_t)(1 << 24) && rows_cap >= 0 && rows_cap <= (int64_t)INT32_MAX - 65536,
+                 "%s: n_expert=%lld rows_cap=%lld", who, (long long)n_expert, (long long)rows_cap);
+    FMOE_REQUIRE((reinterpret_cast<uintptr_t>(dev_tab) & 15u) == 0, "%s: the segment table must be 16-byte aligned", who);
+    prm.dev_tab = dev_tab;
+    prm.dev_rows_cap = rows_cap;
+    prm.tab.n = (int32_t)n_expert;
+    prm.tab.first_expert = 0;
+    return FMOE_OK;
+}
+
 int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
                            int64_t row_hi, hipStream_t stream) {
+    if (a.dev_tab != nullptr) {
+        FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
+                     "linear_forward: in_feat=%lld out_feat=%lld", (long long)a.in_feat, (long long)a.out_feat);
+        if (a.dev_rows_cap == 0) return FMOE_OK;
+        FMOE_REQUIRE(a.x && a.w && a.y, "linear_forward: NULL tensor");
+        const bool fast = is_fast(a.dtype, {a.x, a.w, a.y, a.aux, a.bias}, {a.in_feat, a.out_feat});
+        FMOE_REQUIRE(a.x_row_index == nullptr || linear_forward_can_gather(a),
+                     "linear_forward: rows cannot be gathered in the loader for this shape");
+        const TileShape tile = pick_rows_tile_estimate(a.dev_rows_cap, n_expert, a.out_feat);
+        GemmParams prm{};
+        if (int rc = device_table_launch("linear_forward", prm, a.dev_tab, a.dev_rows_cap, n_expert, fast)) return rc;
+        prm.block_m = tile.bm; prm.block_n = tile.bn;
+        prm.profile_class = kProfGemmFwd; prm.profile_work = 2.0 * (double)a.dev_rows_cap * (double)a.in_feat * (double)a.out_feat;
+        prm.P = a.w; prm.Q = a.x; prm.C = a.y; prm.bias = a.bias; prm.aux = a.aux;
+        prm.q_row_index = a.x_row_index; prm.q_index_div = a.x_index_div; prm.q_total_rows = a.x_total_rows;
+        prm.ldp = a.in_feat; prm.ldq = a.in_feat; prm.ldc = a.out_feat;
+        prm.p_expert_stride = a.in_feat * a.out_feat;
+        prm.bias_expert_stride = a.out_feat;
+        prm.n_cols = (int)a.out_feat; prm.k_extent = (int)a.in_feat;
+        prm.activation = a.activation;
+        return dispatch<kFwd>(prm, a.dtype, a.epilogue, fast, stream);
+    }
     int64_t total;
     if (int rc = check_counts("linear_forward", counts, n_expert, row_lo, row_hi, &total)) return rc;
     FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
@@ -377,6 +421,24 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
 
 int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
                          int64_t row_hi, hipStream_t stream) {
+    if (a.dev_tab != nullptr) {
+        FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
+                     "linear_dgrad: in_feat=%lld out_feat=%lld", (long long)a.in_feat, (long long)a.out_feat);
+        if (a.dev_rows_cap == 0) return FMOE_OK;
+        FMOE_REQUIRE(a.gy && a.w && a.gx, "linear_dgrad: NULL tensor");
+        const bool fast = is_fast(a.dtype, {a.gy, a.w, a.gx, a.aux}, {a.in_feat, a.out_feat});
+        const TileShape tile = pick_rows_tile_estimate(a.dev_rows_cap, n_expert, a.in_feat);
+        GemmParams prm{};
+        if (int rc = device_table_launch("linear_dgrad", prm, a.dev_tab, a.dev_rows_cap, n_expert, fast)) return rc;
+        prm.block_m = tile.bm; prm.block_n = tile.bn;
+        prm.profile_class = kProfGemmDgrad; prm.profile_work = 2.0 * (double)a.dev_rows_cap * (double)a.in_feat * (double)a.out_feat;
+        prm.P = a.w; prm.Q = a.gy; prm.C = a.gx; prm.aux = const_cast<void *>(a.aux);
+        prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
+        prm.p_expert_stride = a.in_feat * a.out_feat;
+        prm.n_cols = (int)a.in_feat; prm.k_extent = (int)a.out_feat;
+        prm.activation = a.activation;
+        return dispatch<kDgrad>(prm, a.dtype, a.epilogue, fast, stream);
+    }
     int64_t total;
     if (int rc = check_counts("linear_dgrad", counts, n_expert, row_lo, row_hi, &total)) return rc;
     FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
@@ -404,6 +466,24 @@ int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts, int64_
 
 int grouped_linear_wgrad(const LinearWgradArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
                          int64_t row_hi, bool last_chunk, hipStream_t stream) {
+    if (a.dev_tab != nullptr) {
+        FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
+                     "linear_wgrad: in_feat=%lld out_feat=%lld", (long long)a.in_feat, (long long)a.out_feat);
+        FMOE_REQUIRE(a.gw && (a.dev_rows_cap == 0 || (a.gy && a.x)), "linear_wgrad: NULL tensor");
+        // (with no rows at all the pointers may be NULL: every expert's contraction is empty and nothing is read)
+        const bool fast = is_fast(a.dtype, {a.gy, a.x, a.gw}, {a.in_feat, a.out_feat});
+        const TileShape tile = pick_wgrad_tile(n_expert, a.out_feat, a.in_feat);
+        GemmParams prm{};
+        if (int rc = device_table_launch("linear_wgrad", prm, a.dev_tab, a.dev_rows_cap, n_expert, fast)) return rc;
+        prm.block_m = tile.bm; prm.block_n = tile.bn;
+        prm.profile_class = kProfGemmWgrad; prm.profile_work = 2.0 * (double)a.dev_rows_cap * (double)a.in_feat * (double)a.out_feat;
+        prm.P = a.x; prm.Q = a.gy; prm.C = a.gw; prm.bias_grad = a.gb;
+        prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
+        prm.c_expert_stride = a.in_feat * a.out_feat;
+        prm.n_cols = (int)a.in_feat; prm.n_rows = (int)a.out_feat;
+        prm.accumulate_first = 0;
+        return dispatch<kWgrad>(prm, a.dtype, kEpiStore, fast, stream);
+    }
     int64_t total;
     if (int rc = check_counts("linear_wgrad", counts, n_expert, row_lo, row_hi, &total)) return rc;
     FMOE_REQUIRE(a.in_feat >= 1 && a.out_feat >= 1 && a.in_feat < (1 << 30) && a.out_feat < (1 << 30),
@@ -528,4 +608,60 @@ extern "C" int fmoe_linear_backward(const void *grad_y, const void *x, const voi
             return rc;
     }
     return FMOE_OK;
+}
+
+// ---- the same products over a segment table in device memory ---------------------------------
+
+extern "C" int fmoe_linear_dev_supported(int64_t in_feat, int64_t out_feat, int dtype) {
+    const int eb = dtype_bytes(dtype);
+    if (eb == 0 || dtype == FMOE_F64 || in_feat < 1 || out_feat < 1) return 0;
+    const int64_t ce = 16 / eb;
+    return (in_feat % ce == 0 && out_feat % ce == 0 && in_feat * eb <= (1 << 22) && out_feat * eb <= (1 << 22)) ? 1 : 0;
+}
+
+extern "C" int fmoe_linear_forward_dev(const void *x, const int64_t *x_row_index, int64_t x_index_div,
+                                       int64_t x_total_rows, const void *w, const void *bias, void *pre, void *y,
+                                       const void *segment_table, int64_t n_expert, int64_t rows_cap, int64_t in_feat,
+                                       int64_t out_feat, int dtype, int activation, void *stream) {
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_forward_dev: unknown dtype %d", dtype);
+    FMOE_REQUIRE(activation >= FMOE_ACT_NONE && activation <= FMOE_ACT_GELU, "fmoe_linear_forward_dev: activation %d",
+                 activation);
+    FMOE_REQUIRE(segment_table != nullptr, "fmoe_linear_forward_dev: NULL segment table");
+    FMOE_REQUIRE(x_row_index == nullptr || (x_index_div >= 1 && x_total_rows >= 0),
+                 "fmoe_linear_forward_dev: x_index_div=%lld x_total_rows=%lld", (long long)x_index_div, (long long)x_total_rows);
+    const bool plain = activation == FMOE_ACT_NONE && pre == nullptr;
+    LinearForwardArgs a{x, w, bias, y, pre, in_feat, out_feat, dtype, plain ? kEpiStore : kEpiBiasAct, activation};
+    a.x_row_index = x_row_index;
+    a.x_index_div = x_row_index ? x_index_div : 1;
+    a.x_total_rows = x_row_index ? x_total_rows : 0;
+    a.dev_tab = (const int32_t *)segment_table;
+    a.dev_rows_cap = rows_cap;
+    return grouped_linear_forward(a, nullptr, n_expert, 0, rows_cap, (hipStream_t)stream);
+}
+
+extern "C" int fmoe_linear_dgrad_dev(const void *grad_y, const void *w, const void *pre, void *grad_x,
+                                     const void *segment_table, int64_t n_expert, int64_t rows_cap, int64_t in_feat,
+                                     int64_t out_feat, int dtype, int activation, void *stream) {
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_dgrad_dev: unknown dtype %d", dtype);
+    FMOE_REQUIRE(activation >= FMOE_ACT_NONE && activation <= FMOE_ACT_GELU, "fmoe_linear_dgrad_dev: activation %d",
+                 activation);
+    FMOE_REQUIRE(segment_table != nullptr, "fmoe_linear_dgrad_dev: NULL segment table");
+    FMOE_REQUIRE(activation == FMOE_ACT_NONE || rows_cap == 0 || pre != nullptr, "fmoe_linear_dgrad_dev: pre is NULL");
+    const bool has_act = activation != FMOE_ACT_NONE;
+    LinearDgradArgs d{grad_y, w, grad_x, has_act ? pre : nullptr, in_feat, out_feat, dtype,
+                      has_act ? kEpiDAct : kEpiStore, activation};
+    d.dev_tab = (const int32_t *)segment_table;
+    d.dev_rows_cap = rows_cap;
+    return grouped_linear_dgrad(d, nullptr, n_expert, 0, rows_cap, (hipStream_t)stream);
+}
+
+extern "C" int fmoe_linear_wgrad_dev(const void *grad_y, const void *x, void *grad_w, void *grad_b,
+                                     const void *segment_table, int64_t n_expert, int64_t rows_cap, int64_t in_feat,
+                                     int64_t out_feat, int dtype, void *stream) {
+    FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_wgrad_dev: unknown dtype %d", dtype);
+    FMOE_REQUIRE(segment_table != nullptr, "fmoe_linear_wgrad_dev: NULL segment table");
+    LinearWgradArgs g{grad_y, x, grad_w, grad_b, in_feat, out_feat, dtype};
+    g.dev_tab = (const int32_t *)segment_table;
+    g.dev_rows_cap = rows_cap;
+    return grouped_linear_wgrad(g, nullptr, n_expert, 0, rows_cap, true, (hipStream_t)stream);
 }

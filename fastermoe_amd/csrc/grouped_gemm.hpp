@@ -24,6 +24,35 @@ struct SegmentTable {
     int32_t tile[kMaxGroupExperts + 1];   // prefix of row tiles (ragged-M launches)
 };
 
+// Segment table in device memory, for launches that must not wait for the expert counts to
+// reach the host: built by segment_table_kernel from the routing's counts, read by the grouped
+// GEMM through scalar loads.  All entries are int32:
+//   [0] n_expert   [1] rows (sum of the counts)   [2] row tiles of 256   [3] row tiles of 128
+//   [4] offset of the 256-row tile map            [5] offset of the 128-row tile map
+//   [6] rows_cap the table was laid out for       [7] 0
+//   [8 .. 8+E]           seg: first row of every expert, seg[E] = rows
+//   [.. +E+1] [.. +E+1]  exclusive prefix of the experts' row tiles, 256 and 128 rows high
+//   tile maps            one {expert, first row, rows, 0} per row tile, 16-byte aligned
+// A launch is sized for the most row tiles `rows_cap` rows can make (rows_cap / BM + E); the
+// workgroups beyond the table's tile count leave at once.
+namespace segtab {
+constexpr int kHeader = 8;
+constexpr int kRows = 1, kTiles256 = 2, kTiles128 = 3, kMap256 = 4, kMap128 = 5, kRowsCap = 6;
+__host__ __device__ inline int64_t cap_tiles(int64_t rows_cap, int64_t n_expert, int block_rows) {
+    return rows_cap / block_rows + (n_expert < rows_cap ? n_expert : rows_cap);
+}
+__host__ __device__ inline int64_t seg_off() { return kHeader; }
+__host__ __device__ inline int64_t pfx256_off(int64_t n_expert) { return kHeader + (n_expert + 1); }
+__host__ __device__ inline int64_t pfx128_off(int64_t n_expert) { return kHeader + 2 * (n_expert + 1); }
+__host__ __device__ inline int64_t map256_off(int64_t n_expert) { return (kHeader + 3 * (n_expert + 1) + 3) / 4 * 4; }
+__host__ __device__ inline int64_t map128_off(int64_t rows_cap, int64_t n_expert) {
+    return map256_off(n_expert) + 4 * cap_tiles(rows_cap, n_expert, 256);
+}
+__host__ __device__ inline int64_t total_ints(int64_t rows_cap, int64_t n_expert) {
+    return map128_off(rows_cap, n_expert) + 4 * cap_tiles(rows_cap, n_expert, 128);
+}
+}  // namespace segtab
+
 struct LinearForwardArgs {
     const void *x;      // [rows, in]; with x_row_index: the token matrix [x_total_rows, in]
     const void *w;      // [E, out, in]
@@ -36,6 +65,10 @@ struct LinearForwardArgs {
     // loader); only honoured where linear_forward_can_gather() says so
     const int64_t *x_row_index = nullptr;
     int64_t x_index_div = 1, x_total_rows = 0;
+    // optional: the segments come from a device table (segtab) laid out for dev_rows_cap rows; the
+    // host counts are then not read (may be NULL) and the row range must be everything
+    const int32_t *dev_tab = nullptr;
+    int64_t dev_rows_cap = 0;
 };
 
 // Whether the forward product can read its rows through an index: the MFMA path (aligned pointers,
@@ -49,6 +82,8 @@ struct LinearDgradArgs {
     const void *aux;    // [rows, in] pre-activation (kEpiDAct) or null
     int64_t in_feat, out_feat;
     int dtype, epilogue, activation;
+    const int32_t *dev_tab = nullptr;  // as in LinearForwardArgs
+    int64_t dev_rows_cap = 0;
 };
 
 struct LinearWgradArgs {
@@ -58,6 +93,8 @@ struct LinearWgradArgs {
     void *gb;           // [E, out] bias gradient (column sums of gy per expert) or null
     int64_t in_feat, out_feat;
     int dtype;
+    const int32_t *dev_tab = nullptr;  // as in LinearForwardArgs
+    int64_t dev_rows_cap = 0;
 };
 
 // counts[e] rows for experts [0, n_expert), restricted to rows [row_lo, row_hi)

@@ -473,6 +473,108 @@ def linear_weight_backward(grad_output_buf, input_buf, expert_count, weight, bia
     return [grad_w, grad_b]
 
 
+# ---- per-expert linear over a segment table in device memory ------------------------------
+
+def segment_table(expert_count, rows_cap):
+    """The row segments of ``expert_count`` (int64 ``[E]``, on the device) as the int32 table the
+    ``*_dev`` products read: built by one small kernel, nothing is read back.  ``rows_cap`` bounds
+    the sum of the counts (counts beyond it are clamped)."""
+    _dev("expert_count", expert_count, torch.int64)
+    lib = _lib.load()
+    n_expert = expert_count.numel()
+    nbytes = lib.fmoe_segment_table_bytes(int(rows_cap), n_expert)
+    with torch.cuda.device(expert_count.device):
+        table = torch.empty(nbytes // 4, dtype=torch.int32, device=expert_count.device)
+        check(lib.fmoe_segment_table_build(_ptr(expert_count), n_expert, int(rows_cap), _ptr(table), nbytes,
+                                           _stream(expert_count)))
+    return table
+
+
+def linear_dev_supported(in_feat, out_feat, dtype):
+    """Whether the ``*_dev`` products take this shape (else: the host-count entry points)."""
+    return dtype in _DTYPES and _lib.load().fmoe_linear_dev_supported(int(in_feat), int(out_feat), _DTYPES[dtype]) == 1
+
+
+def _check_table(table, n_expert, rows_cap):
+    _dev("segment_table", table, torch.int32)
+    need = _lib.load().fmoe_segment_table_bytes(int(rows_cap), int(n_expert)) // 4
+    if table.numel() < need:
+        raise ValueError(f"segment_table has {table.numel()} entries, {need} needed for {rows_cap} rows / {n_expert} experts")
+
+
+def linear_forward_dev(x, weight, bias, table, rows_cap, activation=_lib.ACT_NONE, keep_pre=False,
+                       row_index=None, index_div=1):
+    """``y = act(x @ W_e^T + b_e)`` per expert segment of ``table``; returns ``(y, pre)`` with ``pre``
+    the pre-activation when ``keep_pre``.  With ``row_index`` (int64 ``[rows_cap]``) sorted row ``r`` is
+    read from ``x[row_index[r] // index_div]`` in the GEMM's loader.  Outputs have ``rows_cap`` rows,
+    of which only the table's rows are written."""
+    dt = _rows("x", x)
+    _dev("weight", weight, x.dtype)
+    if weight.dim() != 3 or weight.shape[2] != x.shape[1]:
+        raise ValueError(f"weight must be [num_expert, out_feat, {x.shape[1]}], got {tuple(weight.shape)}")
+    n_expert, out_feat, in_feat = weight.shape
+    if bias is not None:
+        _dev("bias", bias, x.dtype)
+        if tuple(bias.shape) != (n_expert, out_feat):
+            raise ValueError(f"bias must be [{n_expert}, {out_feat}], got {tuple(bias.shape)}")
+    _check_table(table, n_expert, rows_cap)
+    if row_index is not None:
+        _dev("row_index", row_index, torch.int64)
+        if row_index.numel() < rows_cap:
+            raise ValueError("row_index must have one entry per row")
+    elif x.shape[0] < rows_cap:
+        raise ValueError(f"x has {x.shape[0]} rows, rows_cap is {rows_cap}")
+    new = lambda: torch.empty(rows_cap, out_feat, dtype=x.dtype, device=x.device)
+    y = new()
+    pre = new() if keep_pre else None
+    with torch.cuda.device(x.device):
+        check(_lib.load().fmoe_linear_forward_dev(_ptr(x), _ptr(row_index), int(index_div), x.shape[0], _ptr(weight),
+                                                  _ptr(bias), _ptr(pre), _ptr(y), _ptr(table), n_expert, int(rows_cap),
+                                                  in_feat, out_feat, dt, activation, _stream(x)))
+    return y, pre
+
+
+def linear_dgrad_dev(grad_y, weight, table, rows_cap, pre=None, activation=_lib.ACT_NONE):
+    """``(grad_y @ W_e) * act'(pre)`` per expert segment of ``table`` (no activation: the plain
+    data gradient)."""
+    dt = _rows("grad_y", grad_y)
+    _dev("weight", weight, grad_y.dtype)
+    if weight.dim() != 3 or weight.shape[1] != grad_y.shape[1]:
+        raise ValueError(f"weight must be [num_expert, {grad_y.shape[1]}, in_feat], got {tuple(weight.shape)}")
+    n_expert, out_feat, in_feat = weight.shape
+    _check_table(table, n_expert, rows_cap)
+    if grad_y.shape[0] < rows_cap:
+        raise ValueError(f"grad_y has {grad_y.shape[0]} rows, rows_cap is {rows_cap}")
+    if activation != _lib.ACT_NONE:
+        _dev("pre", pre, grad_y.dtype)
+        if pre.dim() != 2 or pre.shape[0] < rows_cap or pre.shape[1] != in_feat:
+            raise ValueError(f"pre must be [>= {rows_cap}, {in_feat}]")
+    grad_x = torch.empty(rows_cap, in_feat, dtype=grad_y.dtype, device=grad_y.device)
+    with torch.cuda.device(grad_y.device):
+        check(_lib.load().fmoe_linear_dgrad_dev(_ptr(grad_y), _ptr(weight),
+                                                _ptr(pre if activation != _lib.ACT_NONE else None), _ptr(grad_x),
+                                                _ptr(table), n_expert, int(rows_cap), in_feat, out_feat, dt, activation,
+                                                _stream(grad_y)))
+    return grad_x
+
+
+def linear_wgrad_dev(grad_y, x, weight, table, rows_cap, with_bias):
+    """``[grad_weight, grad_bias]`` of a per-expert linear over the segments of ``table``
+    (``grad_bias`` is ``None`` unless ``with_bias``); ``weight`` only gives the shape."""
+    dt = _rows("x", x)
+    _dev("grad_y", grad_y, x.dtype)
+    n_expert, out_feat, in_feat = weight.shape
+    if x.shape[1] != in_feat or grad_y.shape[1] != out_feat or x.shape[0] < rows_cap or grad_y.shape[0] < rows_cap:
+        raise ValueError(f"x must be [>= {rows_cap}, {in_feat}] and grad_y [>= {rows_cap}, {out_feat}]")
+    _check_table(table, n_expert, rows_cap)
+    grad_w = torch.empty(n_expert, out_feat, in_feat, dtype=x.dtype, device=x.device)
+    grad_b = torch.empty(n_expert, out_feat, dtype=x.dtype, device=x.device) if with_bias else None
+    with torch.cuda.device(x.device):
+        check(_lib.load().fmoe_linear_wgrad_dev(_ptr(grad_y), _ptr(x), _ptr(grad_w), _ptr(grad_b), _ptr(table), n_expert,
+                                                int(rows_cap), in_feat, out_feat, dt, _stream(x)))
+    return grad_w, grad_b
+
+
 # ---- fused expert MLP (chunked, stream-overlapped pipeline) -------------------------
 
 def _mlp_params(w1, b1, w2, b2, activation):

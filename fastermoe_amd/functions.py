@@ -89,51 +89,40 @@ class _PendingCounts:
     in; it carries this object as ``_fmoe_pending``, and whoever reads its values calls
     :meth:`wait` first (``fmoe_native`` does, just before a launch that needs them), so that all
     host work up to that point runs while the GPU is still busy with whatever precedes the
-    routing, instead of after it."""
+    routing, instead of after it.  Only the fused pipeline of this package's own expert module is
+    handed such a tensor: it goes to the bindings unread."""
 
-    _staging = {}  # (thread, device, n_expert) -> pinned int64 buffer, reused: wait() copies out of it
+    # (thread, device, n_expert) -> [pinned int64 buffer, the _PendingCounts whose copy is in it or None]
+    _staging = {}
 
     def __init__(self, counts):
         import threading
         key = (threading.get_ident(), counts.device.index, counts.numel())
-        buf = self._staging.get(key)
-        if buf is None:
-            buf = self._staging[key] = torch.empty(counts.numel(), dtype=torch.int64, pin_memory=True)
-        self._buf = buf
-        with torch.no_grad():
-            buf.copy_(counts, non_blocking=True)
-        self._event = torch.cuda.Event()
-        self._event.record()
+        slot = self._staging.get(key)
+        if slot is None:
+            slot = self._staging[key] = [torch.empty(counts.numel(), dtype=torch.int64, pin_memory=True), None]
+        elif slot[1] is not None:
+            slot[1].wait()   # an earlier read-back that nobody has waited for yet still owns the buffer
+        self._buf = slot[0]
+        self._slot = slot
         self._done = False
         self.counts_cpu = torch.empty(counts.numel(), dtype=torch.int64)
         self.counts_cpu._fmoe_pending = self
+        # the copy and the event go to the current stream of the counts' device, whichever device is current
+        with torch.cuda.device(counts.device), torch.no_grad():
+            self._buf.copy_(counts, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record(torch.cuda.current_stream(counts.device))
+        slot[1] = self
 
     def wait(self):
         if not self._done:
             self._event.synchronize()
             self.counts_cpu.copy_(self._buf)
             self._done = True
+            if self._slot[1] is self:
+                self._slot[1] = None
         return self.counts_cpu
-
-
-class _ScatterRouted(Function):
-    r"""``MOEScatter`` (fmoe/functions.py:196-248) for rows routed by this package's own routing
-    call, enqueued BEFORE the expert counts are on the host: the gather runs over every entry of
-    ``pos_buf`` (the entries past the routed slots are -1 and give zero rows) and its result, one
-    row per slot with the routed rows first, is returned as it is -- the grouped GEMMs that follow
-    take the counts for how many of its rows to touch."""
-
-    @staticmethod
-    def forward(ctx, inp, pos_buf, slot_to_row, top_k):
-        ctx.moe_args = inp.shape[0], top_k
-        ctx.save_for_backward(slot_to_row)
-        return fmoe_native.gather_rows(inp.contiguous(), pos_buf, index_div=top_k)
-
-    @staticmethod
-    def backward(ctx, grad_buf):
-        (slot_to_row,) = ctx.saved_tensors
-        n_tokens, top_k = ctx.moe_args
-        return fmoe_native.reduce_slots(grad_buf.contiguous(), slot_to_row, n_tokens, top_k), None, None, None
 
 
 def count_by_gate(gate, num_expert, world_size, require_pos=True):
@@ -273,6 +262,49 @@ class MOEExpertMLP(Function):
         gw2, gb2 = fmoe_native.linear_weight_backward(grad_out, mid, fwd_expert_count, w2, b2)
         g_inp, gw1, gb1 = fmoe_native.linear_backward(g_pre, inp, fwd_expert_count, w1, b1)
         return g_inp, None, gw1, gb1, gw2, gb2, None
+
+
+class MOERoutedMLP(Function):
+    r"""``MOEScatter`` -> ``Linear -> activation -> Linear`` (fmoe/functions.py:196-248,
+    fmoe/transformer.py:22-30) over the rows as the routing kernels left them, with nothing read
+    back to the host: the first GEMM reads token row ``pos_buf[r] // top_k`` for sorted row ``r``
+    in its loader (no scattered copy), and all GEMMs take the experts' row segments from
+    ``table``, the device-side segment table of the routing's counts.  Returns the experts' output
+    in expert-sorted order, one row per slot (``[n_slots, d_model]``; the rows past the routed
+    ones are not written), for :class:`MOEGatherCombine` / :class:`MOEGather`.  The backward makes
+    the sorted copy of the input that the first linear's weight gradient contracts over.
+    Not in the reference; same results as ``MOEScatter`` + the three modules."""
+
+    @staticmethod
+    def forward(ctx, inp, w1, b1, w2, b2, pos_buf, slot_to_row, table, top_k, activation):
+        from . import _lib
+        inp = inp.contiguous()
+        n_slots = pos_buf.numel()
+        keep_pre = activation == _lib.ACT_GELU  # ReLU's derivative can be read off the output
+        in_loader = inp.numel() * inp.element_size() < (1 << 31)
+        src = inp if in_loader else fmoe_native.gather_rows(inp, pos_buf, index_div=top_k)
+        mid, pre = fmoe_native.linear_forward_dev(src, w1, b1, table, n_slots, activation, keep_pre,
+                                                  row_index=pos_buf if in_loader else None, index_div=top_k)
+        out, _ = fmoe_native.linear_forward_dev(mid, w2, b2, table, n_slots)
+        ctx.save_for_backward(inp, w1, b1, w2, b2, pos_buf, slot_to_row, table, pre, mid)
+        ctx.moe_args = top_k, activation
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        inp, w1, b1, w2, b2, pos_buf, slot_to_row, table, pre, mid = ctx.saved_tensors
+        top_k, activation = ctx.moe_args
+        n_slots = pos_buf.numel()
+        grad_out = grad_out.contiguous()
+        g_pre = fmoe_native.linear_dgrad_dev(grad_out, w2, table, n_slots, pre if pre is not None else mid, activation)
+        gw2, gb2 = fmoe_native.linear_wgrad_dev(grad_out, mid, w2, table, n_slots, b2 is not None)
+        g_inp = None
+        if ctx.needs_input_grad[0]:
+            g_rows = fmoe_native.linear_dgrad_dev(g_pre, w1, table, n_slots)
+            g_inp = fmoe_native.reduce_slots(g_rows, slot_to_row, inp.shape[0], top_k)
+        rows = fmoe_native.gather_rows(inp, pos_buf, index_div=top_k)
+        gw1, gb1 = fmoe_native.linear_wgrad_dev(g_pre, rows, w1, table, n_slots, b1 is not None)
+        return g_inp, gw1, gb1, gw2, gb2, None, None, None, None, None
 
 
 class MOEGather(Function):

@@ -8,7 +8,7 @@ import torch.nn as nn
 
 from . import fmoe_native
 from .functions import (AllGather, MaskRestore, MaskSelect, MOECache, MOECombine, MOEGather, MOEGatherCombine,
-                        MOELinear, MOEScatter, Slice, _PendingCounts, _ScatterRouted, _prepare_forward_ex, _route_launch,
+                        MOELinear, MOEScatter, Slice, _PendingCounts, _prepare_forward_ex, _route_launch,
                         _single_worker, ensure_comm, mask_index)
 from .gates import NaiveGate
 
@@ -51,6 +51,15 @@ def mark_module_parallel_comm(module, comm):
         setattr(p, "dp_comm", comm)
 
 
+def _own_expert_path(expert_fn, experts):
+    """True when ``expert_fn`` is :meth:`FMoE.expert_fn` itself (not overridden, not replaced on the
+    instance) and ``experts`` is this package's ``_Expert`` with its own ``forward``: only then may
+    the layer skip handing rows and counts through ``expert_fn``."""
+    from .transformer import _Expert
+    return (getattr(expert_fn, "__func__", None) is FMoE.expert_fn
+            and isinstance(experts, _Expert) and type(experts).forward is _Expert.forward)
+
+
 def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_expert, world_size,
                                  fused, enable_fuse=False, combine_score=None):
     r"""Route, scatter, run the experts, gather (fmoe/layers.py:79-149).  Returns
@@ -62,22 +71,32 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
     from .fused_functions import MOEForward
 
     topk = gate.shape[1] if gate.dim() == 2 else 1
-    # Unfused path on the GPU with one gate index per (token, k) pair: the row scatter is enqueued
-    # before the host reads the expert counts (which everything after it needs), so the copy runs
-    # while the host waits for them and prepares the experts' launches.
-    early = (inp.is_cuda and gate.is_cuda and inp.dim() == 2
-             and gate.numel() == inp.shape[0] * topk and inp.shape[0] > 0
-             and (not enable_fuse or combine_score is not None))
-    scattered = None
-    if early:
+    # On the GPU, with one gate index per (token, k) pair and this package's own expert module
+    # behind the layer's own expert_fn, nothing between the gate and the combine needs the expert
+    # counts on the host:
+    #   * unfused: the grouped GEMMs take the row segments from a table the device builds from the
+    #     routing's counts, and the first of them reads the token rows through `pos` in its loader;
+    #   * fused pipeline: the counts are read back asynchronously and waited for inside the
+    #     pipeline call's binding, where the chunk bounds are computed.
+    # Any other expert_fn or expert module gets what the reference gives it: exactly the routed
+    # rows and CPU counts it can read (fmoe/layers.py:117-140).
+    own = (inp.is_cuda and gate.is_cuda and inp.dim() == 2 and inp.shape[0] > 0
+           and gate.numel() == inp.shape[0] * topk and fused and _own_expert_path(expert_fn, experts))
+    if own:
         _single_worker(world_size, "count_by_gate")
         counts_dev, pos_buf, slot_to_row = _route_launch(gate, num_expert)
-        # the counts are read back asynchronously and waited for where their values are first needed
-        # (the binding of the first grouped GEMM, or of the fused pipeline); the sorted buffers of
-        # this path hold one row per slot, the routed rows first
-        counts_cpu = _PendingCounts(counts_dev).counts_cpu
         if not enable_fuse:
-            scattered = _ScatterRouted.apply(inp, pos_buf, slot_to_row, topk)
+            x = experts.routed_forward(inp, pos_buf, slot_to_row, counts_dev, topk)
+            if x is not None:
+                stored_models = torch.zeros(world_size * num_expert, dtype=torch.bool)
+                if combine_score is not None:
+                    return MOEGatherCombine.apply(x, slot_to_row, combine_score, inp.shape[0], topk), stored_models
+                return MOEGather.apply(x, pos_buf, None, None, stored_models, inp.shape[0] * topk, world_size,
+                                       slot_to_row), stored_models
+            own = False
+    if own:
+        # fused pipeline: its sorted buffers hold one row per slot, the routed rows first
+        counts_cpu = _PendingCounts(counts_dev).counts_cpu
         pos = pos_buf
         local_expert_count = global_expert_count = all_expert_count = all_global_expert_count = counts_cpu
         fwd_expert_count = counts_cpu
@@ -108,12 +127,9 @@ def _fmoe_general_global_forward(inp, gate, expert_fn, policy_fn, experts, num_e
 
     # ZeroGate hands back N*top_k indices as a 1-D tensor, so the slot count can
     # exceed the token count; the per-token reduction only applies when it does not.
-    if scattered is not None:
-        x = scattered
-    else:
-        per_token = slot_to_row if slot_to_row.numel() == inp.shape[0] * topk else None
-        x = MOEScatter.apply(inp, pos // topk, local_expert_count, global_expert_count, stored_models,
-                             fwd_batch_size, world_size, per_token, topk)
+    per_token = slot_to_row if slot_to_row.numel() == inp.shape[0] * topk else None
+    x = MOEScatter.apply(inp, pos // topk, local_expert_count, global_expert_count, stored_models,
+                         fwd_batch_size, world_size, per_token, topk)
     x = expert_fn(x, models, fwd_expert_count, num_expert)
     if combine_score is not None:
         return MOEGatherCombine.apply(x, slot_to_row, combine_score, inp.shape[0], topk), stored_models
@@ -175,23 +191,8 @@ class FMoE(nn.Module):
         experts = models[0]
         if not experts:
             raise ValueError(f"Experts is {experts} yet counts is {fwd_expert_count}")
-        if self.experts_fused and getattr(experts[0], "_fmoe_counts_via_bindings", False):
-            # this package's own expert module hands the counts to the grouped-GEMM bindings unread: they
-            # may still be on their way from the device, and ``inp`` may hold one row per slot, of which
-            # the routed ones, as many as the counts add up to, come first
-            # (the very tensor object, not a view of it: the pending read-back rides on it)
-            return experts[0](inp, fwd_expert_count if fwd_expert_count.dim() == 1 else fwd_expert_count.view(-1))
-        pending = getattr(fwd_expert_count, "_fmoe_pending", None)
-        if pending is not None:
-            pending.wait()
         if self.experts_fused:
-            # any other fused expert module gets what the reference gives it: exactly the routed rows
-            # and counts it can read
-            n_rows = int(fwd_expert_count.sum())
-            out = experts[0](inp if n_rows == inp.shape[0] else inp[:n_rows], fwd_expert_count.view(-1))
-            if n_rows == inp.shape[0]:
-                return out
-            return torch.cat([out, out.new_zeros(inp.shape[0] - n_rows, *out.shape[1:])], dim=0)
+            return experts[0](inp, fwd_expert_count.view(-1))
         sizes = [int(n) for n in fwd_expert_count.view(-1).tolist()]
         if sum(sizes) > inp.shape[0]:
             raise ValueError(f"expert counts {sizes} add up to more than the {inp.shape[0]} rows given")

@@ -294,6 +294,64 @@ int fmoe_linear_dact_backward(const void *grad_y, const void *w, const void *pre
                               int64_t out_feat, int dtype, int activation,
                               void *stream);
 
+/* ---- the same products without the expert counts on the host ------------ */
+
+/* The four entry points above read expert_count_host on the host, as
+ * cuda/parallel_linear.cuh:69,85,113 does, so a layer call has to wait for a
+ * device-to-host copy of the counts between its routing kernels and its first
+ * GEMM.  The entry points below take the row segments from a table in DEVICE
+ * memory instead, which one small kernel builds from the counts fmoe_route /
+ * fmoe_gate_topk_route leave on the device; nothing waits for the host and the
+ * whole layer can be captured in a HIP graph.  No counterpart in the reference
+ * (what they replace: the host loops of cuda/parallel_linear.cuh:55-161 and the
+ * .item() / .cpu() reads of fmoe/functions.py:38-40,64-68).
+ *
+ * Bytes of a table for at most rows_cap expert-sorted rows over n_expert experts. */
+int64_t fmoe_segment_table_bytes(int64_t rows_cap, int64_t n_expert);
+
+/* Builds the table from expert_count [n_expert] int64 (device).  Counts are
+ * taken in order and clamped so that they never add up to more than rows_cap
+ * (a count < 0 reads as 0).  segment_table: 16-byte aligned device memory of
+ * fmoe_segment_table_bytes(rows_cap, n_expert) bytes. */
+int fmoe_segment_table_build(const int64_t *expert_count, int64_t n_expert,
+                             int64_t rows_cap, void *segment_table,
+                             int64_t table_bytes, void *stream);
+
+/* 1 when the three entry points below take this shape (16- or 32-bit floats,
+ * feature sizes that are multiples of 16 bytes), else 0.  Host only. */
+int fmoe_linear_dev_supported(int64_t in_feat, int64_t out_feat, int dtype);
+
+/* fmoe_linear_forward / fmoe_linear_act_forward over a device table:
+ *   pre[seg_e] = x[seg_e] . w[e]^T + bias[e]  (stored when pre != NULL)
+ *   y[seg_e]   = act(pre[seg_e])              (activation FMOE_ACT_NONE: y = pre)
+ * x, pre, y have at least rows_cap rows, of which the table's rows are touched.
+ * x_row_index != NULL: expert-sorted row r is read from row
+ * x_row_index[r] / x_index_div of x [x_total_rows, in_feat] instead of row r --
+ * the local scatter (_local_scatter, fmoe/functions.py:72-74) done by the
+ * GEMM's loader, with x_row_index = pos and x_index_div = top_k; x must then
+ * be smaller than 2 GiB. */
+int fmoe_linear_forward_dev(const void *x, const int64_t *x_row_index,
+                            int64_t x_index_div, int64_t x_total_rows,
+                            const void *w, const void *bias, void *pre, void *y,
+                            const void *segment_table, int64_t n_expert,
+                            int64_t rows_cap, int64_t in_feat, int64_t out_feat,
+                            int dtype, int activation, void *stream);
+
+/* Data gradient, as fmoe_linear_dact_backward (activation FMOE_ACT_NONE: the
+ * plain data gradient of fmoe_linear_backward, pre ignored). */
+int fmoe_linear_dgrad_dev(const void *grad_y, const void *w, const void *pre,
+                          void *grad_x, const void *segment_table,
+                          int64_t n_expert, int64_t rows_cap, int64_t in_feat,
+                          int64_t out_feat, int dtype, int activation,
+                          void *stream);
+
+/* Weight and bias gradient, as the grad_w / grad_b half of fmoe_linear_backward
+ * (an expert without rows gets zeros; grad_b may be NULL). */
+int fmoe_linear_wgrad_dev(const void *grad_y, const void *x, void *grad_w,
+                          void *grad_b, const void *segment_table,
+                          int64_t n_expert, int64_t rows_cap, int64_t in_feat,
+                          int64_t out_feat, int dtype, void *stream);
+
 /* How a forward / data-grad launch of `total_tiles` output tiles (256 x 256, or
  * 128 x 256 for small launches) with `contraction_slabs` slabs of 128
  * contraction bytes is spread over `compute_units` (0: the current device's):

@@ -146,9 +146,10 @@ def per_expert_linear(inp_sorted, counts, weight, bias):
 
 
 def time_cpu_baseline(n_tokens, d_model, d_hidden, n_expert, top_k, activation="gelu",
-                      seed=0, repeats=1, threads=None):
-    """Wall-clock fwd+bwd of the brute-force oracle in fp32 on the host cores.
-    Returns (tokens_per_second, cores_used, seconds_per_iteration)."""
+                      seed=0, repeats=1, threads=None, warmup=0, return_median=False):
+    """Wall-clock fwd+bwd of the brute-force oracle in fp32 on the host cores: ``warmup`` untimed
+    iterations, then ``repeats`` timed ones.  Returns (tokens_per_second of the best iteration,
+    cores_used, seconds of the best iteration[, seconds of the median iteration])."""
     import os
     threads = threads or os.cpu_count()
     torch.set_num_threads(threads)
@@ -162,11 +163,15 @@ def time_cpu_baseline(n_tokens, d_model, d_hidden, n_expert, top_k, activation="
     w2 = (torch.rand(n_expert, d_model, d_hidden, generator=g) * 2 - 1) * bound2
     b1 = torch.zeros(n_expert, d_hidden)
     b2 = torch.zeros(n_expert, d_model)
-    best = None
-    for _ in range(repeats):
+    times = []
+    for it in range(warmup + repeats):
         t0 = time.perf_counter()
         moe_mlp_forward_backward(x, idx, score, w1, b1, w2, b2, activation, top_k,
                                  dtype=torch.float32, loss="sum")
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
+        if it >= warmup:
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    best, median = times[0], times[len(times) // 2]
+    if return_median:
+        return n_tokens / best, threads, best, median
     return n_tokens / best, threads, best

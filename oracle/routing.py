@@ -115,6 +115,29 @@ def limit_and_prune(topk_idx, n_expert, capacity):
     return new_lec, new_gec, pruned
 
 
+def segment_table(counts, rows_cap):
+    """The row segments the per-expert GEMMs walk, restated from the host loops of
+    cuda/parallel_linear.cuh:69-88 and :113-155 (``ptr += expert_count[i]`` per expert): expert ``e``
+    owns the expert-sorted rows ``[seg[e], seg[e+1])``.  Beside them, for row tiles of 256 and of
+    128 rows counted from each expert's own first row, the list of ``(expert, first row, rows)``
+    per tile in expert order.  Counts are taken in order and clamped so that they never add up
+    to more than ``rows_cap`` (a negative count reads as 0).  One plain sequential walk."""
+    seg = [0]
+    tiles = {256: [], 128: []}
+    for e, c in enumerate(np.asarray(counts).reshape(-1).tolist()):
+        c = min(max(int(c), 0), rows_cap - seg[-1])
+        first = seg[-1]
+        for block in (256, 128):
+            r = 0
+            while r < c:
+                tiles[block].append((e, first + r, min(block, c - r)))
+                r += block
+        seg.append(first + c)
+    return {"seg": np.array(seg, dtype=np.int32),
+            "tiles256": np.array(tiles[256], dtype=np.int32).reshape(-1, 3),
+            "tiles128": np.array(tiles[128], dtype=np.int32).reshape(-1, 3)}
+
+
 # ---- pure-Python loops, tiny inputs only -----------------------------------
 
 def assign_pos_py(counts, gate):

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in fmoe_hip.h but not exported"
     assert set(declared) == set(_lib.SIGNATURES), "ctypes table and header disagree"
-    assert lib.fmoe_abi_version() == 2
+    assert lib.fmoe_abi_version() == 3
 
 
 def test_ctypes_signatures_match_the_header():

@@ -844,3 +844,119 @@ def test_user_fused_experts_get_the_routed_rows_and_readable_counts(device):
     assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
     out.sum().backward()
     assert torch.allclose(x.grad, (score * scale).sum(dim=1, keepdim=True).expand(n, d), rtol=1e-5, atol=1e-6)
+
+
+def test_replaced_expert_fn_reads_ready_counts(device):
+    """Only FMoE.expert_fn itself is bypassed by the layer's own path over device tables.  An
+    overriding sub-class, or a function assigned on the instance as the reference's tests do
+    (``model.expert_fn = ...``), is called with exactly the routed rows and CPU counts that are
+    there to read, and its result is what the layer returns."""
+    torch.manual_seed(5)
+    n, d, h, e, k = 300, 32, 64, 4, 2
+    seen = []
+
+    class Sub(fmoe.FMoETransformerMLP):
+        def expert_fn(self, inp, models, fwd_expert_count, num_expert):
+            seen.append((inp.shape[0], fwd_expert_count.view(-1).tolist()))
+            return super().expert_fn(inp, models, fwd_expert_count, num_expert)
+
+    idx = torch.randint(-1, e, (n, k), device=device)
+    score = torch.rand(n, k, device=device)
+    want = torch.bincount(idx[idx >= 0].view(-1).cpu(), minlength=e).tolist()
+    x = torch.randn(n, d, device=device)
+    plain = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k).to(device)
+    sub = Sub(num_expert=e, d_model=d, d_hidden=h, top_k=k).to(device)
+    sub.load_state_dict(plain.state_dict())
+    assigned = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k).to(device)
+    assigned.load_state_dict(plain.state_dict())
+    original = assigned.expert_fn
+
+    def replacement(inp, models, fwd_expert_count, num_expert):
+        seen.append((inp.shape[0], [int(c) for c in fwd_expert_count.view(-1, num_expert).sum(0)]))
+        return original(inp, models, fwd_expert_count, num_expert)
+
+    assigned.expert_fn = replacement
+    outs = []
+    for moe in (plain, sub, assigned):
+        moe.gate.forward = lambda inp: (idx, score)
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        out.sum().backward()
+        outs.append((out, xi.grad, moe.experts.htoh4.weight.grad))
+    assert seen == [(sum(want), want), (sum(want), want)]
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert rel_err(a, b) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fold", ["1", "0"])
+def test_unfused_layer_over_device_tables_equals_the_host_count_path(dtype, fold, device, monkeypatch):
+    """The unfused layer's own path (row segments from a device table, token rows read through pos in
+    the first GEMM's loader, no scattered copy, nothing read back) against FMOE_DEVICE_TABLES=0
+    (MOEScatter, host counts, as fmoe/layers.py:117-148): the same products in the same order, so
+    the same bits out of the forward and the same gradients.  Drops, an empty expert, ragged tiles."""
+    torch.manual_seed(78)
+    monkeypatch.setenv("FMOE_FOLD_COMBINE", fold)
+    monkeypatch.setenv("FMOE_GEMM_TILE", "128x128")   # (the two paths pick the tile from different estimates)
+    n, d, h, e, k = 700, 128, 320, 5, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe = moe.to(dtype).to(device)
+    x = torch.randn(n, d).to(dtype).to(device)
+    idx = torch.randint(-1, e - 1, (n, k), device=device)
+    score = torch.rand(n, k, device=device).to(dtype)
+    moe.gate.forward = lambda inp: (idx, score)
+    results = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("FMOE_DEVICE_TABLES", flag)
+        moe.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = moe(xi)
+        out.float().mean().backward()
+        results.append([out, xi.grad] + [p.grad.clone() for p in moe.experts.parameters()])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layer_forward_in_a_hip_graph_with_new_routing_per_replay(dtype, device):
+    """Nothing in the unfused layer's forward waits for the host (the row segments stay on the device),
+    so gate, routing, both grouped GEMMs and the combine can be captured in one HIP graph.  The graph
+    is replayed on inputs that route differently each time (other expert counts, other tile counts),
+    with eager work and synchronisations between the replays; every replay must equal the eager
+    forward on the same input, bit for bit."""
+    torch.manual_seed(9)
+    n, d, h, e, k = 1500, 128, 256, 6, 2
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe = moe.to(dtype).to(device).eval()
+    with torch.no_grad():
+        moe.gate.gate.weight.mul_(30.0)   # well separated logits
+    inputs = [torch.randn(n, d).to(dtype).to(device) for _ in range(4)]
+    # skew the routing differently per input: push the tokens towards one expert's gate row
+    for i, xin in enumerate(inputs):
+        xin[: n // 2] += 0.5 * moe.gate.gate.weight[i % e].detach().to(dtype) / 30.0
+    static_x = inputs[0].clone()
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                moe(static_x)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = moe(static_x)
+        counts_seen = set()
+        for rep in range(6):
+            xin = inputs[rep % len(inputs)]
+            static_x.copy_(xin)
+            graph.replay()
+            torch.cuda.synchronize()
+            got = static_out.clone()
+            want = moe(xin)                     # eager work between the replays
+            idx, _ = moe.gate(xin)
+            counts_seen.add(tuple(torch.bincount(idx.view(-1), minlength=e).tolist()))
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), f"replay {rep}"
+    assert len(counts_seen) >= 3   # the replays really routed differently

@@ -235,3 +235,36 @@ def test_per_expert_backward_matches_autograd(act, bias):
     out.backward(go.double())
     assert torch.allclose(got["grad_inp"], xx.grad, rtol=1e-11, atol=1e-13)
     assert torch.allclose(got["grad_w1"], W1.grad, rtol=1e-11, atol=1e-13)
+
+
+@pytest.mark.parametrize("counts,cap", [([3, 0, 700, 256, 1, 0], 960), ([0, 0, 0], 10), ([5000], 5000),
+                                        ([300, 300, 300], 700), ([-4, 10, 2 ** 40, 7], 100)])
+def test_segment_table_oracle_closed_forms(counts, cap):
+    """Pins oracle.routing.segment_table by what the arithmetic fixes: the segments are the clipped
+    running sums of the (clamped) counts, every expert has ceil(rows / block) tiles, the tiles of an
+    expert tile its segment exactly and in order, and only an expert's last tile may be short."""
+    t = orouting.segment_table(np.array(counts, dtype=np.int64), cap)
+    clamped = np.clip(np.array(counts, dtype=object), 0, None)
+    run = np.minimum(np.concatenate([[0], np.cumsum(clamped)]), cap).astype(np.int64)
+    assert t["seg"].tolist() == run.tolist()
+    rows = np.diff(run)
+    for block, key in ((256, "tiles256"), (128, "tiles128")):
+        tiles = t[key]
+        assert np.array_equal(np.bincount(tiles[:, 0], minlength=len(counts)) if len(tiles) else np.zeros(len(counts), int),
+                              -(-rows // block))
+        assert np.all(np.diff(tiles[:, 0]) >= 0)
+        covered = np.zeros(max(int(run[-1]), 1), dtype=int)
+        for e, first, n in tiles.tolist():
+            assert run[e] <= first and first + n <= run[e + 1] and 1 <= n <= block
+            assert (first - run[e]) % block == 0
+            assert n == block or first + n == run[e + 1]
+            covered[first:first + n] += 1
+        assert np.all(covered[:int(run[-1])] == 1)
+
+
+def test_segment_table_oracle_hand_case():
+    # 3 experts with 300, 0 and 130 rows: expert 0 has a whole 256-row tile and 44 rows more
+    t = orouting.segment_table([300, 0, 130], 1000)
+    assert t["seg"].tolist() == [0, 300, 300, 430]
+    assert t["tiles256"].tolist() == [[0, 0, 256], [0, 256, 44], [2, 300, 130]]
+    assert t["tiles128"].tolist() == [[0, 0, 128], [0, 128, 128], [0, 256, 44], [2, 300, 128], [2, 428, 2]]
