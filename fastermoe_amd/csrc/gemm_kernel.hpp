@@ -185,6 +185,10 @@ struct GemmParams {
     // loader and the sorted copy of the input is never written.
     const int64_t *q_row_index;
     int64_t q_index_div, q_total_rows;
+    // n / q_index_div for 0 <= n < 2^31 as umulhi(n, q_div_mul) >> q_div_shift (q_div_shift < 0: divisor 1);
+    // filled in by set_row_index_divisor()
+    uint32_t q_div_mul;
+    int32_t q_div_shift;
     // Ragged rows only.  The tiles beyond the last whole round of the chip (tiles main_tiles ..
     // total_tiles - 1 of the logical order) can be split along the contraction: k_split
     // workgroups compute split_slabs slabs each and leave their fp32 accumulators in split_ws;
@@ -197,12 +201,26 @@ struct GemmParams {
     // for the most tiles the table can describe, the kernel reads the real counts.  tab.n is then
     // the expert count (any number), tab.first_expert 0, and nothing is split.
     const int32_t *dev_tab;
+    int32_t dev_map_off;       // offset (in int32) of the tile map for this launch's tile height
     int64_t dev_rows_cap;      // host only: rows the device table was laid out for
     int32_t block_m, block_n;  // host only: tile height the segment table was built for (256 or 128) and tile width
     int32_t profile_class;     // host only: ProfileClass of this launch
     double profile_work;       // host only: flop of this launch
     SegmentTable tab;
 };
+
+// Division of a 31-bit number by d through a multiplication: with s = ceil(log2 d) and
+// m = floor(2^(31+s) / d) + 1 (which fits 32 bits for d >= 2), floor(n * m / 2^(31+s)) = floor(n / d) for
+// every 0 <= n < 2^31, because the excess m d - 2^(31+s) is at most d <= 2^s, so the error term
+// n (m d - 2^(31+s)) / (d 2^(31+s)) stays below 1 / d.
+inline void set_row_index_divisor(GemmParams &prm, int64_t divisor) {
+    prm.q_index_div = divisor;
+    if (divisor <= 1) { prm.q_div_mul = 0; prm.q_div_shift = -1; return; }
+    int s = 0;
+    while (((int64_t)1 << s) < divisor) ++s;
+    prm.q_div_mul = (uint32_t)((((uint64_t)1 << (31 + s)) / (uint64_t)divisor) + 1);
+    prm.q_div_shift = s - 1;   // after the multiply-high's shift by 32
+}
 
 // KC slabs: 16-byte chunk c of row r is stored at chunk c ^ swz(r).
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
@@ -296,10 +314,13 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
         if (RAGGED == kRaggedRows) {
             if (dev) {
                 // {expert, first row, rows} of row tile mt
-                const int at = dtab[BM == 256 ? segtab::kMap256 : segtab::kMap128] + 4 * mt;
-                ei = dtab[at];
-                seg_lo = dtab[at + 1];
-                seg_hi = seg_lo + dtab[at + 2];
+                // (the map's offset is known to the host, so this load waits for the tile count only)
+                typedef int i32x4 __attribute__((ext_vector_type(4)));
+                typedef const i32x4 __attribute__((address_space(4))) *DevTab4;
+                const i32x4 entry = *(DevTab4)(dtab + prm.dev_map_off + 4 * mt);
+                ei = entry[0];
+                seg_lo = entry[1];
+                seg_hi = seg_lo + entry[2];
             } else {
                 int lo = 0, hi = prm.tab.n;  // tile[lo] <= mt < tile[hi]
                 while (hi - lo > 1) {
@@ -432,7 +453,14 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
             for (int it = 0; it < NQ; ++it) {
                 const int row = it * kRowsPerPass + r;
                 int64_t src = -1;
-                if (row < q_valid && t < kLoaders) src = prm.q_row_index[q_row0 + row] / prm.q_index_div;
+                if (row < q_valid && t < kLoaders) {
+                    // slot indices fit 31 bits (checked by the host), so idx / q_index_div is a multiply-high and
+                    // a shift by constants the host derived from the divisor (a 64-bit division takes hundreds
+                    // of instructions, and eight of them stood between a tile's start and its first loads)
+                    const int64_t idx = prm.q_row_index[q_row0 + row];
+                    if (idx >= 0 && idx <= (int64_t)INT32_MAX)
+                        src = prm.q_div_shift < 0 ? idx : (int64_t)(__umulhi((uint32_t)idx, prm.q_div_mul) >> prm.q_div_shift);
+                }
                 q_voff[it] = (src >= 0 && src < prm.q_total_rows)
                                  ? (uint32_t)((src * prm.ldq + q_kc_chunk * CE) * (int64_t)sizeof(T))
                                  : kOutOfRange;
@@ -1171,6 +1199,8 @@ int launch_for_height(GemmParams &prm, int epi, hipStream_t stream) {
         prm.tiles_m = 0;
         // device table: the most row tiles its rows can make (the kernel drops the surplus workgroups)
         total = (prm.dev_tab ? segtab::cap_tiles(prm.dev_rows_cap, prm.tab.n, BM) : (int64_t)prm.tab.tile[prm.tab.n]) * prm.tiles_n;
+        if (prm.dev_tab)
+            prm.dev_map_off = (int32_t)(BM == 256 ? segtab::map256_off(prm.tab.n) : segtab::map128_off(prm.dev_rows_cap, prm.tab.n));
     } else {
         prm.tiles_m = (int)ceil_div(prm.n_rows, BM);
         total = (int64_t)prm.tab.n * prm.tiles_m * prm.tiles_n;

@@ -348,7 +348,11 @@ float *split_workspace(hipStream_t stream, size_t bytes) {
 bool linear_forward_can_gather(const LinearForwardArgs &a) {
     if (a.dtype == FMOE_F64 || dtype_bytes(a.dtype) == 0) return false;
     if (!is_fast(a.dtype, {a.x, a.w, a.y, a.aux, a.bias}, {a.in_feat, a.out_feat})) return false;
-    return a.x_total_rows >= 0 && a.x_total_rows * a.in_feat * (int64_t)dtype_bytes(a.dtype) < ((int64_t)1 << 31);
+    // (the loader divides 31-bit indices: every index that names a row must fit)
+    if (a.x_index_div < 1 || a.x_index_div > (int64_t)INT32_MAX || a.x_total_rows < 0 ||
+        a.x_total_rows > (int64_t)INT32_MAX / a.x_index_div)
+        return false;
+    return a.x_total_rows * a.in_feat * (int64_t)dtype_bytes(a.dtype) < ((int64_t)1 << 31);
 }
 
 // checks shared by the launches over a device table; fills the parts of prm that say so
@@ -382,7 +386,7 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
         prm.block_m = tile.bm; prm.block_n = tile.bn;
         prm.profile_class = kProfGemmFwd; prm.profile_work = 2.0 * (double)a.dev_rows_cap * (double)a.in_feat * (double)a.out_feat;
         prm.P = a.w; prm.Q = a.x; prm.C = a.y; prm.bias = a.bias; prm.aux = a.aux;
-        prm.q_row_index = a.x_row_index; prm.q_index_div = a.x_index_div; prm.q_total_rows = a.x_total_rows;
+        prm.q_row_index = a.x_row_index; set_row_index_divisor(prm, a.x_index_div); prm.q_total_rows = a.x_total_rows;
         prm.ldp = a.in_feat; prm.ldq = a.in_feat; prm.ldc = a.out_feat;
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.bias_expert_stride = a.out_feat;
@@ -408,7 +412,7 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
         fill_table(&prm.tab, counts, e0, e1, row_lo, row_hi, tile.bm);
         prm.profile_class = kProfGemmFwd; prm.profile_work = table_flop(prm.tab, a.in_feat, a.out_feat);
         prm.P = a.w; prm.Q = a.x; prm.C = a.y; prm.bias = a.bias; prm.aux = a.aux;
-        prm.q_row_index = a.x_row_index; prm.q_index_div = a.x_index_div; prm.q_total_rows = a.x_total_rows;
+        prm.q_row_index = a.x_row_index; set_row_index_divisor(prm, a.x_index_div); prm.q_total_rows = a.x_total_rows;
         prm.ldp = a.in_feat; prm.ldq = a.in_feat; prm.ldc = a.out_feat;
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.bias_expert_stride = a.out_feat;
