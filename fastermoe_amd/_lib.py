@@ -33,6 +33,9 @@ SIGNATURES = {
     "fmoe_route": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp]),
     "fmoe_route_static": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp]),
     "fmoe_gate_topk_route": (_int, [_vp, _i64, _i64, _i64, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "fmoe_gate_linear_supported": (_int, [_i64, _i64, _i64, _int]),
+    "fmoe_gate_linear_topk_route": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp,
+                                           _i64, _vp]),
     "fmoe_gate_topk_backward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     "fmoe_limit_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "fmoe_prune_gate_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp]),

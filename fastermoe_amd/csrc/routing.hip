@@ -19,6 +19,7 @@
 #include "common.hpp"
 
 #include <mutex>
+#include <type_traits>
 
 namespace fmoe {
 namespace {
@@ -269,6 +270,24 @@ __global__ __launch_bounds__(kBlock) void rank_apply_kernel(
 
 // ----------------------------------------------------------------- gate ----
 
+// Keeps the K largest (value, expert) pairs seen so far in descending order of the value.  A
+// later value only displaces a strictly smaller one, so ties go to the lower expert index; a
+// place that is still empty (idx < 0) takes anything, so a row with fewer than K values above
+// -inf still names K experts (torch.topk, which this stands in for, does too; unlike torch.topk,
+// which ranks NaN above everything, a NaN is taken as -inf here).
+template <int K>
+__device__ __forceinline__ void topk_insert(float (&val)[K], int (&idx)[K], float x, int e) {
+    x = x != x ? -__builtin_inff() : x;   // a NaN ranks (and scores) as -inf
+#pragma unroll
+    for (int j = K - 1; j >= 0; --j) {
+        const int up = j > 0 ? j - 1 : 0;
+        const bool here = x > val[j] || idx[j] < 0;                   // x belongs at or above place j
+        const bool above = j > 0 && (x > val[up] || idx[up] < 0);      // ... above it: place j takes its upper neighbour
+        val[j] = here ? (above ? val[up] : x) : val[j];
+        idx[j] = here ? (above ? idx[up] : e) : idx[j];
+    }
+}
+
 // Top-k of the gate logits, the scores of the selected experts and the per-workgroup expert
 // histogram that the routing scan starts from, in one pass over the logits.
 //
@@ -299,15 +318,7 @@ __global__ __launch_bounds__(kBlock) void gate_topk_hist_kernel(
         int idx[K];
 #pragma unroll
         for (int j = 0; j < K; ++j) { val[j] = kLowest; idx[j] = -1; }
-        auto insert = [&](float x, int e) {
-#pragma unroll
-            for (int j = K - 1; j >= 0; --j) {
-                const bool here = x > val[j];                       // x belongs at or above place j
-                const bool above = j > 0 && x > val[j > 0 ? j - 1 : 0];  // ... above it: place j takes its upper neighbour
-                val[j] = here ? (above ? val[j > 0 ? j - 1 : 0] : x) : val[j];
-                idx[j] = here ? (above ? idx[j > 0 ? j - 1 : 0] : e) : idx[j];
-            }
-        };
+        auto insert = [&](float x, int e) { topk_insert<K>(val, idx, x, e); };
         if (live) {
             const T *row = logits + token * n_expert;
             int e = 0;
@@ -348,6 +359,158 @@ __global__ __launch_bounds__(kBlock) void gate_topk_hist_kernel(
 #pragma unroll
         for (int w = 0; w < kWavesPerBlock; ++w) c += bins[w * n_expert + e];
         dst[e] = c;
+    }
+}
+
+// The gate's linear layer, its top-k and the scores in one kernel, for up to 64 experts: the logits
+// x W^T + b (fmoe/gates/naive_gate.py:26-31) are formed in registers and LDS and never written
+// to memory.  A workgroup owns kGateTokens tokens; its four waves split the contraction (wave w
+// takes the steps w, w + 4, ... of 128 bytes per row) and feed the MFMA straight from global
+// memory -- for the 16 x 16 block shapes a lane's operand is 16 contiguous bytes of one row of W
+// (expert lb of a 16-expert block) or of x (token lb of a 16-token block), so there is no staging
+// -- then leave their partial [expert][token] tiles in LDS.  Thread t < kGateTokens adds the four
+// partials of its token's logits in wave order (a fixed order), adds the bias, rounds to the
+// element type (what the layer's own output would have been) and keeps the K largest exactly as
+// gate_topk_hist_kernel does.  The routing histogram is left to the routing kernels that follow:
+// the contraction wants many small workgroups, the histogram few large ones.
+constexpr int kGateTokens = 32, kGateMaxExpert = 64, kGateStride = kGateTokens + 4;
+
+template <typename T, int K, int kEB>
+__global__ __launch_bounds__(kBlock) void gate_linear_topk_kernel(
+    const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, int64_t n_tokens, int d,
+    int n_expert, int score_mode, int64_t *__restrict__ topk_idx, T *__restrict__ topk_score) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    extern __shared__ float part_lds[];   // [kWavesPerBlock][16 n_eb][kGateStride]
+    constexpr int kTB = kGateTokens / 16;   // kEB: 16-expert blocks this instantiation holds accumulators for
+    constexpr int kPer = 16 / (int)sizeof(T);       // elements per 16-byte operand
+    constexpr int kStep = 8 * kPer;                 // contraction elements per step of a wave (128 bytes per row)
+    const int lane = lane_id(), wave = threadIdx.x / kWave, lb = lane & 15, hq = lane >> 4;
+    const int64_t token0 = (int64_t)blockIdx.x * kGateTokens;
+    const int n_eb = (n_expert + 15) / 16;
+
+    f32x4 acc[kEB][kTB];
+#pragma unroll
+    for (int eb = 0; eb < kEB; ++eb)
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb) acc[eb][tb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const T *wrow[kEB];
+    const T *xrow[kTB];
+    bool wok[kEB], xok[kTB];
+#pragma unroll
+    for (int eb = 0; eb < kEB; ++eb) {
+        wok[eb] = eb * 16 + lb < n_expert;
+        wrow[eb] = w + (int64_t)(wok[eb] ? eb * 16 + lb : 0) * d;
+    }
+#pragma unroll
+    for (int tb = 0; tb < kTB; ++tb) {
+        xok[tb] = token0 + tb * 16 + lb < n_tokens;
+        xrow[tb] = x + (xok[tb] ? token0 + tb * 16 + lb : 0) * d;
+    }
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 zero4 = {0, 0, 0, 0};
+    auto mma = [&](const u32x4 (&a)[kEB], const u32x4 (&b)[kTB]) {
+#pragma unroll
+        for (int eb = 0; eb < kEB; ++eb) {
+            if (eb >= n_eb) continue;
+#pragma unroll
+            for (int tb = 0; tb < kTB; ++tb) {
+                if constexpr (sizeof(T) == 4) {
+                    const float *af = (const float *)&a[eb], *bf = (const float *)&b[tb];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[eb][tb] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j], bf[j], acc[eb][tb], 0, 0, 0);
+                } else if constexpr (std::is_same<T, __bf16>::value) {
+                    acc[eb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[eb]), __builtin_bit_cast(bf16x8, b[tb]), acc[eb][tb], 0, 0, 0);
+                } else {
+                    acc[eb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[eb]), __builtin_bit_cast(f16x8, b[tb]), acc[eb][tb], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // rows outside the problem read row 0 (and are dropped at the end): no bounds checks on the way.
+    // A wave's step covers 128 bytes of every row -- whole cache lines, as two 64-byte halves (the
+    // operands of two products) -- and the four waves take the steps in turn.
+    constexpr int kUnroll = 2, kStride = kWavesPerBlock * kStep;
+    // Workgroups start at different places of the contraction and wrap around: in step with each
+    // other they would all ask for the same columns of their rows at the same time, which lie a whole
+    // row length apart and so fall on a few memory channels.  (The order of the fp32 additions
+    // then depends on where in the batch a token stands; the result stays a fixed function of the input.)
+    const int n_groups = (d + kUnroll * kStride - 1) / (kUnroll * kStride);
+    const int first = (int)((blockIdx.x * 7u) % (unsigned)n_groups);
+    for (int gi = 0; gi < n_groups; ++gi) {
+        const int g = gi + first < n_groups ? gi + first : gi + first - n_groups;
+        const int k0 = g * (kUnroll * kStride) + wave * kStep;
+        if (k0 + (kUnroll - 1) * kStride + kStep <= d) {
+            // a whole group of kUnroll steps: every load goes out before the first product needs one
+            u32x4 a[kUnroll][2][kEB], b[kUnroll][2][kTB];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const int k = k0 + u * kStride + (c * 4 + hq) * kPer;
+#pragma unroll
+                    for (int tb = 0; tb < kTB; ++tb) b[u][c][tb] = *(const u32x4 *)(xrow[tb] + k);
+#pragma unroll
+                    for (int eb = 0; eb < kEB; ++eb) a[u][c][eb] = eb < n_eb ? *(const u32x4 *)(wrow[eb] + k) : zero4;
+                }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) mma(a[u][c], b[u][c]);
+        } else {
+            for (int ks = k0; ks < d && ks < k0 + kUnroll * kStride; ks += kStride) {
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const int k = ks + (c * 4 + hq) * kPer;   // d is a multiple of kPer: a chunk lies inside the row or outside it
+                    u32x4 a[kEB], b[kTB];
+#pragma unroll
+                    for (int tb = 0; tb < kTB; ++tb) b[tb] = k < d ? *(const u32x4 *)(xrow[tb] + k) : zero4;
+#pragma unroll
+                    for (int eb = 0; eb < kEB; ++eb) a[eb] = (eb < n_eb && k < d) ? *(const u32x4 *)(wrow[eb] + k) : zero4;
+                    mma(a, b);
+                }
+            }
+        }
+    }
+    // lane (lb, hq) holds, per block pair, experts 4 hq .. 4 hq + 3 of the expert block for token lb of the token block
+#pragma unroll
+    for (int eb = 0; eb < kEB; ++eb)
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (eb < n_eb) part_lds[((wave * n_eb + eb) * 16 + 4 * hq + r) * kGateStride + tb * 16 + lb] = acc[eb][tb][r];
+    __syncthreads();
+
+    const int t = threadIdx.x;
+    const int64_t token = token0 + t;
+    if (t >= kGateTokens || token >= n_tokens) return;
+    float val[K];
+    int idx[K];
+#pragma unroll
+    for (int j = 0; j < K; ++j) { val[j] = -__builtin_inff(); idx[j] = -1; }
+    for (int e = 0; e < n_expert; ++e) {
+        const float *p = part_lds + e * kGateStride + t;
+        const int ws = n_eb * 16 * kGateStride;   // one wave's tile
+        float logit = ((p[0] + p[ws]) + p[2 * ws]) + p[3 * ws];
+        if (bias != nullptr) logit += (float)bias[e];
+        topk_insert<K>(val, idx, (float)(T)logit, e);
+    }
+    float score[K];
+#pragma unroll
+    for (int j = 0; j < K; ++j) score[j] = val[j];
+    if (score_mode == 1) {
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < K; ++j) { score[j] = idx[j] >= 0 ? __expf(val[j] - val[0]) : 0.f; sum += score[j]; }
+#pragma unroll
+        for (int j = 0; j < K; ++j) score[j] /= sum;
+    }
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        topk_idx[token * K + j] = idx[j];
+        topk_score[token * K + j] = (T)(idx[j] >= 0 ? score[j] : 0.f);
     }
 }
 
@@ -687,6 +850,81 @@ extern "C" int fmoe_gate_topk_route(const void *logits, int64_t n_tokens, int64_
         topk_idx, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, ilog2_ceil(n_expert), 1);
     FMOE_LAUNCH_CHECK();
     return FMOE_OK;
+}
+
+namespace fmoe {
+namespace {
+
+template <typename T>
+int launch_gate_linear(const void *x, const void *w, const void *bias, int64_t n_tokens, int d, int E, int top_k,
+                       int score_mode, int64_t *topk_idx, void *topk_score, hipStream_t st) {
+    const unsigned grid = (unsigned)ceil_div(n_tokens, kGateTokens);
+    const size_t lds = (size_t)kWavesPerBlock * ((E + 15) / 16 * 16) * kGateStride * sizeof(float);
+    // (accumulators for 1, 2 or 4 blocks of 16 experts: fewer registers, more waves per compute unit)
+#define FMOE_GATE_LINEAR_LAUNCH(KK)                                                                                         \
+    do {                                                                                                                    \
+        if (E <= 16)                                                                                                        \
+            gate_linear_topk_kernel<T, KK, 1><<<grid, kBlock, lds, st>>>((const T *)x, (const T *)w, (const T *)bias,        \
+                                                                         n_tokens, d, E, score_mode, topk_idx, (T *)topk_score); \
+        else if (E <= 32)                                                                                                   \
+            gate_linear_topk_kernel<T, KK, 2><<<grid, kBlock, lds, st>>>((const T *)x, (const T *)w, (const T *)bias,        \
+                                                                         n_tokens, d, E, score_mode, topk_idx, (T *)topk_score); \
+        else                                                                                                                \
+            gate_linear_topk_kernel<T, KK, 4><<<grid, kBlock, lds, st>>>((const T *)x, (const T *)w, (const T *)bias,        \
+                                                                         n_tokens, d, E, score_mode, topk_idx, (T *)topk_score); \
+    } while (0)
+    switch (top_k) {
+        case 1: FMOE_GATE_LINEAR_LAUNCH(1); break;
+        case 2: FMOE_GATE_LINEAR_LAUNCH(2); break;
+        case 4: FMOE_GATE_LINEAR_LAUNCH(4); break;
+        case 8: FMOE_GATE_LINEAR_LAUNCH(8); break;
+        default: return fail(FMOE_ELIMIT, "gate linear top-k: top_k=%d is not 1, 2, 4 or 8", top_k);
+    }
+#undef FMOE_GATE_LINEAR_LAUNCH
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+}  // namespace
+}  // namespace fmoe
+
+extern "C" int fmoe_gate_linear_supported(int64_t d_model, int64_t n_expert, int64_t top_k, int dtype) {
+    if (dtype != FMOE_F32 && dtype != FMOE_BF16 && dtype != FMOE_F16) return 0;
+    if (n_expert < 1 || n_expert > kGateMaxExpert || top_k > n_expert) return 0;
+    if (top_k != 1 && top_k != 2 && top_k != 4 && top_k != 8) return 0;
+    return (d_model >= 1 && d_model < (1 << 30) && (d_model * dtype_bytes(dtype)) % 16 == 0) ? 1 : 0;
+}
+
+extern "C" int fmoe_gate_linear_topk_route(const void *x, const void *w, const void *bias, int64_t n_tokens,
+                                           int64_t d_model, int64_t n_expert, int64_t top_k, int dtype, int score_mode,
+                                           int64_t *topk_idx, void *topk_score, int64_t *expert_count, int64_t *pos,
+                                           int64_t *slot_to_row, void *workspace, int64_t workspace_bytes,
+                                           void *stream) {
+    FMOE_REQUIRE(n_tokens >= 0 && top_k >= 1, "fmoe_gate_linear_topk_route: n_tokens=%lld top_k=%lld",
+                 (long long)n_tokens, (long long)top_k);
+    FMOE_REQUIRE(score_mode == 0 || score_mode == 1, "fmoe_gate_linear_topk_route: score_mode %d", score_mode);
+    if (!fmoe_gate_linear_supported(d_model, n_expert, top_k, dtype))
+        return fail(FMOE_ELIMIT,
+                    "fmoe_gate_linear_topk_route: d_model=%lld n_expert=%lld top_k=%lld dtype=%d is not taken (at most %d "
+                    "experts, top_k 1, 2, 4 or 8, rows of whole 16-byte chunks, 16- or 32-bit floats)",
+                    (long long)d_model, (long long)n_expert, (long long)top_k, dtype, kGateMaxExpert);
+    const int64_t n_slots = n_tokens * top_k;
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    FMOE_REQUIRE(expert_count, "fmoe_gate_linear_topk_route: NULL expert_count");
+    hipStream_t st = (hipStream_t)stream;
+    if (n_slots == 0) return route_empty(n_expert, expert_count, st);
+    FMOE_REQUIRE(x && w && topk_idx && topk_score && pos, "fmoe_gate_linear_topk_route: NULL pointer");
+    FMOE_REQUIRE(aligned16(x) && aligned16(w), "fmoe_gate_linear_topk_route: x and w must be 16-byte aligned");
+    RouteScratch s;
+    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+    int rc = FMOE_OK;
+    switch (dtype) {
+        case FMOE_F32: rc = launch_gate_linear<float>(x, w, bias, n_tokens, (int)d_model, (int)n_expert, (int)top_k, score_mode, topk_idx, topk_score, st); break;
+        case FMOE_BF16: rc = launch_gate_linear<__bf16>(x, w, bias, n_tokens, (int)d_model, (int)n_expert, (int)top_k, score_mode, topk_idx, topk_score, st); break;
+        default: rc = launch_gate_linear<_Float16>(x, w, bias, n_tokens, (int)d_model, (int)n_expert, (int)top_k, score_mode, topk_idx, topk_score, st); break;
+    }
+    if (rc) return rc;
+    return route_launch(topk_idx, n_slots, n_expert, expert_count, pos, slot_to_row, s, st);
 }
 
 extern "C" int fmoe_gate_topk_backward(const void *grad_score, const void *score, const int64_t *topk_idx,

@@ -143,6 +143,43 @@ def gate_topk_route(logits, top_k, score_mode=0):
     return idx, score, cnt, pos, s2r
 
 
+def gate_linear_supported(d_model, n_expert, top_k, dtype):
+    """Whether :func:`gate_linear_topk_route` takes this gate (else: the linear layer and :func:`gate_topk_route`)."""
+    return dtype in _DTYPES and _lib.load().fmoe_gate_linear_supported(int(d_model), int(n_expert), int(top_k),
+                                                                       _DTYPES[dtype]) == 1
+
+
+def gate_linear_topk_route(x, weight, bias, top_k, score_mode=0):
+    """``gate_topk_route(x @ weight.T + bias, ...)`` without the logits ever reaching memory: the gate's
+    linear layer, its top-k, the scores and the routing in one call.  ``weight`` is ``[E, d_model]``
+    (``nn.Linear.weight``), ``bias`` ``[E]`` or ``None``.  Same results tuple as :func:`gate_topk_route`."""
+    dt = _rows("x", x)
+    _dev("weight", weight, x.dtype)
+    if weight.dim() != 2 or weight.shape[1] != x.shape[1]:
+        raise ValueError(f"weight must be [n_expert, {x.shape[1]}], got {tuple(weight.shape)}")
+    n, d = x.shape
+    e = weight.shape[0]
+    if bias is not None:
+        _dev("bias", bias, x.dtype)
+        if tuple(bias.shape) != (e,):
+            raise ValueError(f"bias must be [{e}], got {tuple(bias.shape)}")
+    if not gate_linear_supported(d, e, top_k, x.dtype):
+        raise ValueError(f"gate_linear_topk_route does not take d_model={d}, n_expert={e}, top_k={top_k}, dtype={x.dtype}")
+    lib = _lib.load()
+    dev = x.device
+    with torch.cuda.device(dev):
+        idx = torch.empty(n, top_k, dtype=torch.int64, device=dev)
+        score = torch.empty(n, top_k, dtype=x.dtype, device=dev)
+        cnt = torch.empty(e, dtype=torch.int64, device=dev)
+        pos = torch.empty(n * top_k, dtype=torch.int64, device=dev)
+        s2r = torch.empty(n * top_k, dtype=torch.int64, device=dev)
+        ws = _workspace(lib.fmoe_routing_workspace_bytes(n * top_k, e), dev)
+        check(lib.fmoe_gate_linear_topk_route(_ptr(x), _ptr(weight), _ptr(bias), n, d, e, top_k, dt, score_mode, _ptr(idx),
+                                              _ptr(score), _ptr(cnt), _ptr(pos), _ptr(s2r), _ptr(ws), ws.numel(),
+                                              _stream(x)))
+    return idx, score, cnt, pos, s2r
+
+
 def gate_topk_backward(grad_score, score, topk_idx, n_expert, score_mode=0):
     """Gradient of the top-k scores with respect to the logits, ``[N, E]``."""
     _dev("grad_score", grad_score)

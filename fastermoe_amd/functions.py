@@ -47,6 +47,48 @@ class GateTopK(Function):
         return fmoe_native.gate_topk_backward(grad_score.contiguous(), score, idx, n_expert, score_mode), None, None
 
 
+class GateLinearTopK(Function):
+    r"""``nn.Linear`` -> ``torch.topk`` (-> softmax) of fmoe/gates/naive_gate.py:26-42 and the routing of
+    ``count_by_gate`` in one call that keeps the logits on chip.  Returns ``(topk_idx, topk_score)`` like
+    :class:`GateTopK`; the routing rides on ``topk_idx``.  Backward: the sparse gradient of the logits
+    (``fmoe_gate_topk_backward``), then the linear layer's own backward as two skinny library products."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, top_k, score_mode):
+        x = x.contiguous()
+        weight = weight.contiguous()
+        idx, score, cnt, pos_buf, s2r = fmoe_native.gate_linear_topk_route(x, weight, bias, top_k, score_mode)
+        ctx.save_for_backward(x, weight, idx, score)
+        ctx.moe_args = score_mode, bias is not None
+        ctx.mark_non_differentiable(idx)
+        idx._fmoe_route = (idx._version, weight.shape[0], cnt, pos_buf, s2r)
+        return idx, score
+
+    @staticmethod
+    def backward(ctx, _grad_idx, grad_score):
+        x, weight, idx, score = ctx.saved_tensors
+        score_mode, has_bias = ctx.moe_args
+        g = fmoe_native.gate_topk_backward(grad_score.contiguous(), score, idx, weight.shape[0], score_mode)
+        grad_x = g @ weight if ctx.needs_input_grad[0] else None
+        grad_w = g.t() @ x if ctx.needs_input_grad[1] else None
+        grad_b = g.float().sum(dim=0).to(g.dtype) if has_bias and ctx.needs_input_grad[2] else None
+        return grad_x, grad_w, grad_b, None, None
+
+
+def gate_linear_topk(x, linear, top_k, score_mode=0):
+    r"""Top-k indices and scores of ``linear(x)`` for an ``nn.Linear`` gate: one fused call when the
+    shape is taken (CUDA tensors, at most 64 experts, ``top_k`` 1, 2, 4 or 8, rows of whole 16-byte
+    chunks; ``FMOE_GATE_LINEAR_FUSED=0`` switches it off), else the layer followed by :func:`gate_topk`."""
+    import os
+    w, b = linear.weight, linear.bias
+    if (x.is_cuda and x.dim() == 2 and w.is_cuda and w.dtype == x.dtype and (b is None or b.dtype == x.dtype)
+            and os.environ.get("FMOE_GATE_LINEAR_FUSED", "1") != "0"
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and fmoe_native.gate_linear_supported(x.shape[1], w.shape[0], top_k, x.dtype)):
+        return GateLinearTopK.apply(x, w, b, top_k, score_mode)
+    return gate_topk(linear(x), top_k, score_mode)
+
+
 def gate_topk(logits, top_k, score_mode=0):
     r"""Top-k indices and scores of ``logits [N, E]``: the HIP gate kernel when it takes the shape
     (CUDA tensor, 16/32-bit floats, ``top_k`` 1, 2, 4 or 8), ``torch.topk``

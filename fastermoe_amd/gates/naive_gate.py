@@ -1,7 +1,7 @@
 r"""Top-k of a linear layer (fmoe/gates/naive_gate.py:11-42)."""
 import torch.nn as nn
 
-from ..functions import gate_topk
+from ..functions import gate_linear_topk, gate_topk
 from .base_gate import BaseGate
 
 
@@ -16,11 +16,13 @@ class NaiveGate(BaseGate):
         self.top_k = top_k
 
     def forward(self, inp, return_all_scores=False):
-        logits = self.gate(inp)
         # torch.topk(sorted=False) in the reference; here one kernel that also leaves the expert
         # histogram and the positions for the layer's routing step (order of the k choices: by logit)
-        top_idx, top_val = gate_topk(logits, self.top_k)
-        top_val = top_val.view(-1, self.top_k)
         if return_all_scores:
-            return top_idx, top_val, logits
-        return top_idx, top_val
+            logits = self.gate(inp)
+            top_idx, top_val = gate_topk(logits, self.top_k)
+            return top_idx, top_val.view(-1, self.top_k), logits
+        # nobody asks for the logits: for small expert counts the linear layer runs inside the same
+        # kernel and they never reach memory
+        top_idx, top_val = gate_linear_topk(inp, self.gate, self.top_k)
+        return top_idx, top_val.view(-1, self.top_k)

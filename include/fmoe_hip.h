@@ -114,6 +114,28 @@ int fmoe_gate_topk_route(const void *logits, int64_t n_tokens, int64_t n_expert,
                          int64_t *slot_to_row, void *workspace,
                          int64_t workspace_bytes, void *stream);
 
+/* The gate's linear layer folded into the same call, for small expert counts:
+ * logits = x . w^T + bias are formed on chip (rounded to the element type as the
+ * layer's output would be) and never written to memory; top-k, scores and
+ * routing as above.  x [n_tokens, d_model], w [n_expert, d_model], bias
+ * [n_expert] or NULL, all of `dtype`; x and w 16-byte aligned.
+ * fmoe_gate_linear_supported says whether the shape is taken (at most 64
+ * experts, top_k 1, 2, 4 or 8, d_model a whole number of 16-byte chunks);
+ * FMOE_ELIMIT otherwise.  Replaces nn.Linear + torch.topk (+ softmax) of
+ * fmoe/gates/naive_gate.py:26-42 followed by count_by_gate,
+ * fmoe/functions.py:19-42.  Its backward is fmoe_gate_topk_backward followed by
+ * the linear layer's own (two skinny library GEMMs). */
+int fmoe_gate_linear_supported(int64_t d_model, int64_t n_expert, int64_t top_k,
+                               int dtype);
+int fmoe_gate_linear_topk_route(const void *x, const void *w, const void *bias,
+                                int64_t n_tokens, int64_t d_model,
+                                int64_t n_expert, int64_t top_k, int dtype,
+                                int score_mode, int64_t *topk_idx,
+                                void *topk_score, int64_t *expert_count,
+                                int64_t *pos, int64_t *slot_to_row,
+                                void *workspace, int64_t workspace_bytes,
+                                void *stream);
+
 /* Gradient of topk_score with respect to the logits, [n_tokens, n_expert]
  * (zero at experts that were not selected); score is only read in score_mode 1.
  * Replaces autograd's backward of torch.topk / softmax in the gate. */

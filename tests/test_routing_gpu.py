@@ -11,6 +11,7 @@ from fastermoe_amd import fmoe_native
 from fastermoe_amd.functions import count_by_gate, prepare_forward
 from fastermoe_amd.gates.utils import limit_by_capacity
 from oracle import routing as orouting
+from helpers import TOL, rel_err
 
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "routing_cases.json")
@@ -266,4 +267,128 @@ def test_naive_gate_hands_its_routing_to_the_layer(device):
     val2.sum().backward()
     assert gate.gate.weight.grad is not None and torch.isfinite(gate.gate.weight.grad).all()
     logits = gate.gate(x)
-    assert torch.equal(val2, torch.gather(logits, 1, idx2))
+    # (the gate's linear layer ran inside the top-k kernel: same logits up to the order of the fp32 sums)
+    assert torch.allclose(val2, torch.gather(logits, 1, idx2), rtol=1e-5, atol=1e-5)
+
+
+def test_gate_topk_with_masked_out_logits(device):
+    """Logits of -inf (experts masked out by a caller) and NaN: a token with fewer than top_k finite
+    logits still names top_k distinct experts -- the finite ones first, then the lowest-numbered of
+    the rest -- instead of -1, which the gates would feed to bincount / index_add."""
+    from fastermoe_amd import fmoe_native
+    ninf = float("-inf")
+    logits = torch.tensor([[ninf, 2.0, ninf, ninf, 1.0, ninf],
+                           [ninf, ninf, ninf, ninf, ninf, ninf],
+                           [0.5, ninf, 3.0, float("nan"), ninf, -1.0]], device=device)
+    idx, score, cnt, pos_buf, s2r = fmoe_native.gate_topk_route(logits, 4, 0)
+    assert idx.cpu().tolist() == [[1, 4, 0, 2], [0, 1, 2, 3], [2, 0, 5, 1]]
+    assert score[0, :2].cpu().tolist() == [2.0, 1.0] and torch.isinf(score[0, 2:]).all()
+    ref_pos, ref_cnt = orouting.count_by_gate(idx.cpu().numpy(), 6)
+    assert np.array_equal(cnt.cpu().numpy(), ref_cnt) and int(ref_cnt.sum()) == 12
+    assert np.array_equal(pos_buf.cpu().numpy(), ref_pos)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,d,e,k,bias", [
+    (32768, 4096, 8, 2, True),     # the Mixtral-like share's gate
+    (4096, 512, 8, 2, True),       # the tiny fp32 layer's gate
+    (16384, 2048, 64, 1, True),    # top-1 over 64 experts
+    (16384, 1024, 16, 2, False),
+    (1000, 72, 5, 4, True),        # experts not a multiple of 16, tokens not a multiple of a workgroup's share,
+                                   # contraction not a multiple of a wave's step
+    (33, 8, 2, 2, True),
+    (100, 264, 64, 8, True),
+    (0, 64, 4, 2, True),
+])
+def test_gate_linear_topk_route(dtype, n, d, e, k, bias, device):
+    """The gate's linear layer inside the top-k kernel (fmoe_gate_linear_topk_route) against
+    nn.Linear + torch.topk: the logits, formed in float64 from the same operands and rounded to the
+    element type, fix the selection for every token whose k+1 largest logits are further apart than
+    the rounding of the two different summation orders can move them -- those tokens must match
+    torch.topk exactly; the scores must be the (rounded) logits of whatever was selected; and the
+    routing must be the oracle's on the same index tensor, bit for bit."""
+    from fastermoe_amd import fmoe_native
+    gen = torch.Generator().manual_seed(n + d + e)
+    x = torch.randn(n, d, generator=gen).to(dtype)
+    w = (torch.randn(e, d, generator=gen) * (3.0 / d ** 0.5)).to(dtype)
+    b = torch.randn(e, generator=gen).to(dtype) if bias else None
+    xd, wd, bd = x.to(device), w.to(device), (b.to(device) if bias else None)
+    ref = x.double() @ w.double().t()
+    if bias:
+        ref = ref + b.double()
+    for mode in (0, 1):
+        idx, score, cnt, pos_buf, s2r = fmoe_native.gate_linear_topk_route(xd, wd, bd, k, mode)
+        assert idx.shape == (n, k) and score.dtype == dtype
+        ref_pos, ref_cnt = orouting.count_by_gate(idx.cpu().numpy(), e)
+        assert np.array_equal(cnt.cpu().numpy(), ref_cnt) and int(ref_cnt.sum()) == n * k
+        assert np.array_equal(pos_buf.cpu().numpy(), ref_pos)
+        inv = np.full(n * k, -1, dtype=np.int64)
+        inv[ref_pos] = np.arange(n * k)
+        assert np.array_equal(s2r.cpu().numpy(), inv)
+        if n == 0:
+            continue
+        got_idx = idx.cpu()
+        assert (got_idx.sort(dim=1).values.diff(dim=1) > 0).all() if k > 1 else True   # distinct experts
+        top_val, top_idx = torch.topk(ref, min(k + 1, e), dim=1, sorted=True)
+        # (float32: the two fp32 summation orders differ by about sqrt(d) roundings of the partial sums)
+        step = {torch.float32: 2.0 ** -22 * max(1.0, d ** 0.5), torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[dtype]
+        # choice j of a token is settled when its logit is clear of both neighbours in the sorted order
+        gaps = top_val[:, :-1] - top_val[:, 1:]                                   # [n, k] (or [n, e-1])
+        ok = gaps > 4 * step * top_val.abs().max(dim=1, keepdim=True).values.clamp(min=1.0)
+        below = ok if ok.shape[1] == k else torch.cat([ok, torch.ones(n, 1, dtype=torch.bool)], dim=1)
+        above = torch.cat([torch.ones(n, 1, dtype=torch.bool), ok[:, :k - 1]], dim=1)
+        clear = above & below[:, :k]
+        assert clear.float().mean() > 0.3
+        assert torch.equal(got_idx[clear], top_idx[:, :k][clear])
+        picked = torch.gather(ref, 1, got_idx)
+        if mode == 0:
+            want = picked
+        else:
+            want = torch.softmax(picked, dim=1)
+        tol = {torch.float32: 1e-5, torch.bfloat16: 1.6e-2, torch.float16: 2e-3}[dtype]
+        assert torch.allclose(score.double().cpu(), want, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_gate_linear_topk_autograd(dtype, mode, device):
+    """GateLinearTopK's backward against autograd through nn.Linear, a gather at the SAME indices
+    and the softmax: gradients of the input, the weight and the bias."""
+    from fastermoe_amd.functions import GateLinearTopK
+    torch.manual_seed(12)
+    n, d, e, k = 600, 96, 12, 4
+    lin = torch.nn.Linear(d, e).to(dtype).to(device)
+    x = torch.randn(n, d, device=device).to(dtype).requires_grad_(True)
+    g = torch.randn(n, k, device=device).to(dtype)
+    idx, score = GateLinearTopK.apply(x, lin.weight, lin.bias, k, mode)
+    assert hasattr(idx, "_fmoe_route")
+    (score * g).sum().backward()
+    got = [x.grad.clone(), lin.weight.grad.clone(), lin.bias.grad.clone()]
+    x64 = x.detach().double().requires_grad_(True)
+    w64, b64 = lin.weight.detach().double().requires_grad_(True), lin.bias.detach().double().requires_grad_(True)
+    val = torch.gather(x64 @ w64.t() + b64, 1, idx)
+    sc = torch.softmax(val, dim=1) if mode == 1 else val
+    (sc * g.double()).sum().backward()
+    tol = TOL[dtype] if dtype != torch.float32 else 1e-5
+    for a, r in zip(got, [x64.grad, w64.grad, b64.grad]):
+        assert rel_err(a, r) <= tol
+
+
+def test_naive_gate_uses_the_fused_linear_and_matches_the_unfused_one(device, monkeypatch):
+    from fastermoe_amd.gates import NaiveGate
+    torch.manual_seed(4)
+    gate = NaiveGate(256, 16, 1, top_k=2).to(device)
+    x = torch.randn(3000, 256, device=device)
+    results = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("FMOE_GATE_LINEAR_FUSED", flag)
+        gate.zero_grad()
+        idx, val = gate(x)
+        val.square().sum().backward()
+        results.append((idx, val, gate.gate.weight.grad.clone(), gate.gate.bias.grad.clone()))
+    assert torch.equal(results[0][0], results[1][0])            # random fp32 logits: no near-ties
+    for a, b in zip(results[0][1:], results[1][1:]):
+        assert torch.allclose(a, b, rtol=1e-4, atol=1e-4)
+    # with all logits asked for, the gate runs the linear layer by itself
+    idx3, val3, logits = gate(x, return_all_scores=True)
+    assert logits.shape == (3000, 16) and torch.equal(idx3, results[1][0])
