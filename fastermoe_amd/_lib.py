@@ -37,6 +37,10 @@ SIGNATURES = {
     "fmoe_gate_linear_topk_route": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp,
                                            _i64, _vp]),
     "fmoe_gate_topk_backward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
+    "fmoe_noisy_gate_forward": (_int, [_vp, _vp, _vp, ctypes.c_double, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _vp,
+                                       _vp, _vp, _vp, _vp, _i64, _vp]),
+    "fmoe_noisy_gate_backward": (_int, [_vp, _vp, _vp, ctypes.c_double, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _vp,
+                                        _vp, _vp, _vp, _vp]),
     "fmoe_limit_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "fmoe_prune_gate_by_capacity": (_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp]),
     "fmoe_gather_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),

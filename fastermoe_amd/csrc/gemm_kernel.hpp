@@ -137,7 +137,9 @@ __device__ __forceinline__ float gelu_grad_16bit(float x) {
     r = fmaf(r, u, 5.860928472e-02f);
     r = fmaf(r, u, -2.649256521e-01f);
     r = fmaf(r, u, 7.976261318e-01f);
-    return fmaf(xc, r, 0.5f);
+    // (the clamp drops a NaN; x * 0 puts it back, and gives NaN for an infinite pre-activation as
+    // Phi(x) + x phi(x) evaluated literally does: a forward that overflowed still shows in the gradients)
+    return fmaf(x, 0.f, fmaf(xc, r, 0.5f));
 }
 
 // kNarrow: the result is rounded to a 16-bit type

@@ -514,6 +514,162 @@ __global__ __launch_bounds__(kBlock) void gate_linear_topk_kernel(
     }
 }
 
+// ----------------------------------------------------------- noisy gate ----
+
+// Noisy top-k gating (Shazeer et al. 2017, sec. 2.1 and appendix A; fmoe/gates/noisy_gate.py:113-144)
+// in training mode, one pass over the two logit matrices and the noise:
+//   std_e   = softplus(raw_e) + eps            noisy_e = clean_e + noise_e * std_e
+//   v_0 >= ... >= v_K : the K + 1 largest noisy logits (ties to the lower expert), experts i_0 .. i_K
+//   gates_j = softmax(v_0 .. v_{K-1})_j
+//   P_e     = Phi((clean_e - (noisy_e > v_K ? v_K : v_{K-1})) / std_e)      load_e = sum over tokens of P_e
+// A workgroup owns the same kSlotsPerBlock / K tokens as in gate_topk_hist_kernel and leaves the
+// routing histogram of its selections for route_scan_kernel.  The load is summed without atomics:
+// a wave adds its 64 tokens' P_e by a butterfly of lane exchanges, wave-private LDS tables take
+// the sums, the four tables are added in wave order and written per workgroup; the caller adds
+// the workgroups' rows.  thr_val / thr_idx keep (v_{K-1}, v_K) and (i_{K-1}, i_K) for the backward.
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(__expf(x)); }
+__device__ __forceinline__ float normal_cdf_f(float z) { return 0.5f * (1.f + erff(z * 0.70710678118654752440f)); }
+
+template <typename T, int K>
+__global__ __launch_bounds__(kBlock) void noisy_gate_forward_kernel(
+    const T *__restrict__ clean, const T *__restrict__ raw, const T *__restrict__ noise, float eps, int64_t n_tokens,
+    int n_expert, int64_t *__restrict__ topk_idx, T *__restrict__ gates, float *__restrict__ thr_val,
+    int32_t *__restrict__ thr_idx, float *__restrict__ load_partial, int32_t *__restrict__ block_hist, int nbits) {
+    extern __shared__ int32_t bins[];  // [kWavesPerBlock][n_expert] int32 histogram, then the same of float load sums
+    const int wave = threadIdx.x / kWave;
+    int32_t *mine = bins + wave * n_expert;
+    float *loads = (float *)(bins + kWavesPerBlock * n_expert);
+    float *my_load = loads + wave * n_expert;
+    for (int e = threadIdx.x; e < kWavesPerBlock * n_expert; e += kBlock) { bins[e] = 0; loads[e] = 0.f; }
+    __syncthreads();
+
+    constexpr int kTokensPerBlock = kSlotsPerBlock / K, kTokensPerThread = kTokensPerBlock / kBlock;
+    for (int it = 0; it < kTokensPerThread; ++it) {
+        const int64_t token = (int64_t)blockIdx.x * kTokensPerBlock + it * kBlock + threadIdx.x;
+        const bool live = token < n_tokens;
+        const int64_t row = (live ? token : 0) * n_expert;
+        float val[K + 1];
+        int idx[K + 1];
+#pragma unroll
+        for (int j = 0; j <= K; ++j) { val[j] = -__builtin_inff(); idx[j] = -1; }
+        for (int e = 0; e < n_expert; ++e) {
+            const float std_e = softplus_f((float)raw[row + e]) + eps;
+            topk_insert<K + 1>(val, idx, (float)clean[row + e] + (float)noise[row + e] * std_e, e);
+        }
+        float g[K], sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < K; ++j) { g[j] = __expf(val[j] - val[0]); sum += g[j]; }
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                topk_idx[token * K + j] = idx[j];
+                gates[token * K + j] = (T)(g[j] / sum);
+            }
+            thr_val[token * 2] = val[K - 1];
+            thr_val[token * 2 + 1] = val[K];
+            thr_idx[token * 2] = idx[K - 1];
+            thr_idx[token * 2 + 1] = idx[K];
+        }
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+            wave_bins_add(mine, live ? idx[j] : 0, live, match_mask(live ? idx[j] : 0, live, nbits));
+        // the smooth load: every lane's P_e, added over the wave
+        for (int e = 0; e < n_expert; ++e) {
+            float p = 0.f;
+            if (live) {
+                const float c = (float)clean[row + e];
+                const float std_e = softplus_f((float)raw[row + e]) + eps;
+                // (an expert is inside when it is one of the K selected: the same rule as the selection's
+                // under ties, and independent of how the compiler contracts the two evaluations of noisy)
+                bool inside = false;
+#pragma unroll
+                for (int j = 0; j < K; ++j) inside |= idx[j] == e;
+                p = normal_cdf_f((c - (inside ? val[K] : val[K - 1])) / std_e);
+            }
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) p += __shfl_xor(p, off, kWave);
+            if (lane_id() == 0) my_load[e] += p;
+        }
+        wave_lds_sync();
+    }
+    __syncthreads();
+    int32_t *dst = block_hist + (int64_t)blockIdx.x * n_expert;
+    float *ldst = load_partial + (int64_t)blockIdx.x * n_expert;
+    for (int e = threadIdx.x; e < n_expert; e += kBlock) {
+        int32_t c = 0;
+        float l = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) { c += bins[w * n_expert + e]; l += loads[w * n_expert + e]; }
+        dst[e] = c;
+        ldst[e] = l;
+    }
+}
+
+// Backward of the above with respect to the two logit matrices.  Per token, with
+// gg_j the gradient of gates_j (the caller has added the importance term) and gl_e that of load_e:
+//   d noisy_{i_j} = gates_j (gg_j - sum_i gg_i gates_i)                                      (j < K)
+//   dP_e = gl_e phi(z_e):   d clean_e += dP_e / std_e,   d std_e -= dP_e z_e / std_e,
+//                           d noisy_{i_K} -= dP_e / std_e (e inside the top K), d noisy_{i_{K-1}} -= ... (outside)
+//   d clean_e += d noisy_e,  d std_e += d noisy_e noise_e,  d raw_e = d std_e sigmoid(raw_e)
+template <typename T, int K>
+__global__ __launch_bounds__(kBlock) void noisy_gate_backward_kernel(
+    const T *__restrict__ clean, const T *__restrict__ raw, const T *__restrict__ noise, float eps, int64_t n_tokens,
+    int n_expert, const int64_t *__restrict__ topk_idx, const T *__restrict__ gates, const float *__restrict__ thr_val,
+    const int32_t *__restrict__ thr_idx, const T *__restrict__ grad_gates, const float *__restrict__ grad_load,
+    T *__restrict__ grad_clean, T *__restrict__ grad_raw) {
+    const int64_t token = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (token >= n_tokens) return;
+    const int64_t row = token * n_expert;
+    const float v_out = thr_val[token * 2], v_in = thr_val[token * 2 + 1];
+    const int i_out = thr_idx[token * 2], i_in = thr_idx[token * 2 + 1];
+    // the gates again in float32 from the selected experts' noisy logits (the stored ones are rounded
+    // to the element type, and gg_j - sum_i gg_i gates_i cancels when one gate is close to 1)
+    int sel[K];
+    float gt[K], dn[K], dot = 0.f, vmax = -__builtin_inff(), gsum = 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        sel[j] = (int)topk_idx[token * K + j];
+        const int e = sel[j] >= 0 && sel[j] < n_expert ? sel[j] : 0;
+        gt[j] = (float)clean[row + e] + (float)noise[row + e] * (softplus_f((float)raw[row + e]) + eps);
+        vmax = fmaxf(vmax, gt[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < K; ++j) { gt[j] = __expf(gt[j] - vmax); gsum += gt[j]; }
+#pragma unroll
+    for (int j = 0; j < K; ++j) { gt[j] /= gsum; dot += (float)grad_gates[token * K + j] * gt[j]; }
+#pragma unroll
+    for (int j = 0; j < K; ++j) dn[j] = gt[j] * ((float)grad_gates[token * K + j] - dot);
+    // first pass: what the thresholds collect from every expert's load term
+    float s_in = 0.f, s_out = 0.f;
+    for (int e = 0; e < n_expert; ++e) {
+        const float c = (float)clean[row + e];
+        const float std_e = softplus_f((float)raw[row + e]) + eps;
+        bool inside = false;
+#pragma unroll
+        for (int j = 0; j < K; ++j) inside |= sel[j] == e;
+        const float z = (c - (inside ? v_in : v_out)) / std_e;
+        const float dp = grad_load[e] * 0.39894228040143267794f * __expf(-0.5f * z * z) / std_e;
+        if (inside) s_in -= dp; else s_out -= dp;
+    }
+    for (int e = 0; e < n_expert; ++e) {
+        const float c = (float)clean[row + e], r = (float)raw[row + e], nz = (float)noise[row + e];
+        const float std_e = softplus_f(r) + eps;
+        bool inside = false;
+#pragma unroll
+        for (int j = 0; j < K; ++j) inside |= sel[j] == e;
+        const float z = (c - (inside ? v_in : v_out)) / std_e;
+        const float dp = grad_load[e] * 0.39894228040143267794f * __expf(-0.5f * z * z) / std_e;
+        float d_noisy = 0.f;
+#pragma unroll
+        for (int j = 0; j < K; ++j) d_noisy += sel[j] == e ? dn[j] : 0.f;
+        if (e == i_in) d_noisy += s_in;
+        if (e == i_out) d_noisy += s_out;
+        const float d_std = -dp * z + d_noisy * nz;
+        grad_clean[row + e] = (T)(dp + d_noisy);
+        grad_raw[row + e] = (T)(d_std / (1.f + __expf(-r)));
+    }
+}
+
 // Gradient of the scores with respect to the logits: zero except at the selected experts.
 // score_mode 0: grad_logits[t, idx[t,j]] = grad_score[t,j];
 // score_mode 1: grad_logits[t, idx[t,j]] = score[t,j] * (grad_score[t,j] - sum_i grad_score[t,i] score[t,i]).
@@ -570,10 +726,31 @@ int ilog2_ceil(int64_t n) {
     return b < 1 ? 1 : b;
 }
 
-// Dynamic LDS beyond 64 KiB (more than 4096 experts) has to be allowed per kernel.
+// Dynamic LDS beyond 64 KiB (more than 4096 experts) has to be allowed per kernel and device.  The
+// opt-in is made once per (kernel, device) and size reached, outside the launch path of later calls
+// (so that it does not land inside a stream capture); a failure is reported again by every call.
 int allow_lds(const void *kernel, size_t bytes) {
     if (bytes <= 64 * 1024) return FMOE_OK;
-    FMOE_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    struct Granted { const void *kernel; int device; size_t bytes; bool failed; };
+    static std::mutex mutex;
+    static Granted granted[64];
+    static int n_granted = 0;
+    int dev = 0;
+    FMOE_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mutex);
+    Granted *slot = nullptr;
+    for (int i = 0; i < n_granted; ++i)
+        if (granted[i].kernel == kernel && granted[i].device == dev) slot = &granted[i];
+    if (slot != nullptr && !slot->failed && slot->bytes >= bytes) return FMOE_OK;
+    if (slot == nullptr) {
+        FMOE_REQUIRE(n_granted < 64, "too many (kernel, device) pairs ask for more than 64 KiB of LDS");
+        slot = &granted[n_granted++];
+        *slot = Granted{kernel, dev, 0, false};
+    }
+    const hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    slot->failed = err != hipSuccess;
+    if (!slot->failed) slot->bytes = bytes;
+    FMOE_HIP_CHECK(err);
     return FMOE_OK;
 }
 
@@ -925,6 +1102,97 @@ extern "C" int fmoe_gate_linear_topk_route(const void *x, const void *w, const v
     }
     if (rc) return rc;
     return route_launch(topk_idx, n_slots, n_expert, expert_count, pos, slot_to_row, s, st);
+}
+
+extern "C" int fmoe_noisy_gate_forward(const void *clean, const void *raw, const void *noise, double eps,
+                                       int64_t n_tokens, int64_t n_expert, int64_t top_k, int dtype,
+                                       int64_t *topk_idx, void *gates, float *thr_val, int32_t *thr_idx,
+                                       float *load_partial, int64_t *expert_count, int64_t *pos, int64_t *slot_to_row,
+                                       void *workspace, int64_t workspace_bytes, void *stream) {
+    FMOE_REQUIRE(n_tokens >= 0 && top_k >= 1, "fmoe_noisy_gate_forward: n_tokens=%lld top_k=%lld", (long long)n_tokens,
+                 (long long)top_k);
+    FMOE_REQUIRE(dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16, "fmoe_noisy_gate_forward: dtype %d", dtype);
+    if (top_k >= n_expert || (top_k != 1 && top_k != 2 && top_k != 4 && top_k != 8) || n_expert > 2048)
+        return fail(FMOE_ELIMIT, "fmoe_noisy_gate_forward: top_k=%lld must be 1, 2, 4 or 8 and below n_expert=%lld <= 2048",
+                    (long long)top_k, (long long)n_expert);
+    const int64_t n_slots = n_tokens * top_k;
+    if (int rc = check_sizes(n_slots, n_expert)) return rc;
+    FMOE_REQUIRE(expert_count && load_partial, "fmoe_noisy_gate_forward: NULL expert_count / load_partial");
+    hipStream_t st = (hipStream_t)stream;
+    if (n_slots == 0) return route_empty(n_expert, expert_count, st);
+    FMOE_REQUIRE(clean && raw && noise && topk_idx && gates && thr_val && thr_idx && pos,
+                 "fmoe_noisy_gate_forward: NULL pointer");
+    RouteScratch s;
+    if (int rc = carve(workspace, workspace_bytes, n_slots, n_expert, &s)) return rc;
+    const int E = (int)n_expert, nbits = ilog2_ceil(n_expert);
+    const size_t lds = 2 * kWavesPerBlock * E * sizeof(int32_t);
+#define FMOE_NOISY_FWD(TT, KK)                                                                                          \
+    do {                                                                                                                \
+        if (int rc = allow_lds((const void *)noisy_gate_forward_kernel<TT, KK>, lds)) return rc;                        \
+        noisy_gate_forward_kernel<TT, KK><<<s.n_blocks, kBlock, lds, st>>>(                                             \
+            (const TT *)clean, (const TT *)raw, (const TT *)noise, (float)eps, n_tokens, E, topk_idx, (TT *)gates,      \
+            thr_val, thr_idx, load_partial, s.block_hist, nbits);                                                       \
+    } while (0)
+#define FMOE_NOISY_FWD_K(TT)                                                 \
+    switch (top_k) {                                                         \
+        case 1: FMOE_NOISY_FWD(TT, 1); break;                                \
+        case 2: FMOE_NOISY_FWD(TT, 2); break;                                \
+        case 4: FMOE_NOISY_FWD(TT, 4); break;                                \
+        default: FMOE_NOISY_FWD(TT, 8); break;                               \
+    }
+    switch (dtype) {
+        case FMOE_F32: FMOE_NOISY_FWD_K(float); break;
+        case FMOE_BF16: FMOE_NOISY_FWD_K(__bf16); break;
+        default: FMOE_NOISY_FWD_K(_Float16); break;
+    }
+#undef FMOE_NOISY_FWD_K
+#undef FMOE_NOISY_FWD
+    FMOE_LAUNCH_CHECK();
+    route_scan_kernel<<<1, kRouteScanBlock, 0, st>>>(s.block_hist, s.n_blocks, E, expert_count, s.cum);
+    FMOE_LAUNCH_CHECK();
+    if (int rc2 = allow_lds((const void *)rank_apply_kernel<kApplyAssign>, kWavesPerBlock * E * sizeof(int32_t))) return rc2;
+    rank_apply_kernel<kApplyAssign><<<s.n_blocks, kBlock, kWavesPerBlock * E * sizeof(int32_t), st>>>(
+        topk_idx, s.block_hist, s.cum, pos, slot_to_row, n_slots, n_slots, E, nbits, 1);
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_noisy_gate_backward(const void *clean, const void *raw, const void *noise, double eps,
+                                        int64_t n_tokens, int64_t n_expert, int64_t top_k, int dtype,
+                                        const int64_t *topk_idx, const void *gates, const float *thr_val,
+                                        const int32_t *thr_idx, const void *grad_gates, const float *grad_load,
+                                        void *grad_clean, void *grad_raw, void *stream) {
+    FMOE_REQUIRE(n_tokens >= 0 && n_expert >= 1, "fmoe_noisy_gate_backward: bad sizes");
+    FMOE_REQUIRE(dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16, "fmoe_noisy_gate_backward: dtype %d", dtype);
+    if (top_k >= n_expert || (top_k != 1 && top_k != 2 && top_k != 4 && top_k != 8))
+        return fail(FMOE_ELIMIT, "fmoe_noisy_gate_backward: top_k=%lld", (long long)top_k);
+    if (n_tokens == 0) return FMOE_OK;
+    FMOE_REQUIRE(clean && raw && noise && topk_idx && gates && thr_val && thr_idx && grad_gates && grad_load &&
+                     grad_clean && grad_raw, "fmoe_noisy_gate_backward: NULL pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned grid = (unsigned)ceil_div(n_tokens, kBlock);
+    const int E = (int)n_expert;
+#define FMOE_NOISY_BWD(TT, KK)                                                                                            \
+    noisy_gate_backward_kernel<TT, KK><<<grid, kBlock, 0, st>>>((const TT *)clean, (const TT *)raw, (const TT *)noise,   \
+                                                               (float)eps, n_tokens, E, topk_idx, (const TT *)gates,    \
+                                                               thr_val, thr_idx, (const TT *)grad_gates, grad_load,     \
+                                                               (TT *)grad_clean, (TT *)grad_raw)
+#define FMOE_NOISY_BWD_K(TT)                                                 \
+    switch (top_k) {                                                         \
+        case 1: FMOE_NOISY_BWD(TT, 1); break;                                \
+        case 2: FMOE_NOISY_BWD(TT, 2); break;                                \
+        case 4: FMOE_NOISY_BWD(TT, 4); break;                                \
+        default: FMOE_NOISY_BWD(TT, 8); break;                               \
+    }
+    switch (dtype) {
+        case FMOE_F32: FMOE_NOISY_BWD_K(float); break;
+        case FMOE_BF16: FMOE_NOISY_BWD_K(__bf16); break;
+        default: FMOE_NOISY_BWD_K(_Float16); break;
+    }
+#undef FMOE_NOISY_BWD_K
+#undef FMOE_NOISY_BWD
+    FMOE_LAUNCH_CHECK();
+    return FMOE_OK;
 }
 
 extern "C" int fmoe_gate_topk_backward(const void *grad_score, const void *score, const int64_t *topk_idx,

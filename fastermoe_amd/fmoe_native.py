@@ -180,6 +180,58 @@ def gate_linear_topk_route(x, weight, bias, top_k, score_mode=0):
     return idx, score, cnt, pos, s2r
 
 
+def noisy_gate_supported(n_expert, top_k, dtype):
+    """Whether :func:`noisy_gate_forward` takes this gate shape."""
+    return top_k in (1, 2, 4, 8) and top_k < n_expert <= 2048 and dtype in (torch.float32, torch.bfloat16, torch.float16)
+
+
+def noisy_gate_forward(clean, raw, noise, top_k, eps):
+    """Noisy top-k gating after the two linear products (training mode).  Returns ``(topk_idx [N,k],
+    gates [N,k], load float32 [E], thr_val, thr_idx, expert_count, pos_buf, slot_to_row)``;
+    ``thr_val`` / ``thr_idx`` are what :func:`noisy_gate_backward` needs."""
+    dt = _rows("clean", clean)
+    _dev("raw", raw, clean.dtype)
+    _dev("noise", noise, clean.dtype)
+    if raw.shape != clean.shape or noise.shape != clean.shape:
+        raise ValueError("clean, raw and noise must have the same shape [n_tokens, n_expert]")
+    n, e = clean.shape
+    if not noisy_gate_supported(e, top_k, clean.dtype):
+        raise ValueError(f"noisy_gate_forward does not take n_expert={e}, top_k={top_k}, dtype={clean.dtype}")
+    lib = _lib.load()
+    dev = clean.device
+    n_blocks = max(1, -(-n * top_k // 2048))
+    with torch.cuda.device(dev):
+        idx = torch.empty(n, top_k, dtype=torch.int64, device=dev)
+        gates = torch.empty(n, top_k, dtype=clean.dtype, device=dev)
+        thr_val = torch.empty(n, 2, dtype=torch.float32, device=dev)
+        thr_idx = torch.empty(n, 2, dtype=torch.int32, device=dev)
+        partial = torch.zeros(n_blocks, e, dtype=torch.float32, device=dev)
+        cnt = torch.empty(e, dtype=torch.int64, device=dev)
+        pos = torch.empty(n * top_k, dtype=torch.int64, device=dev)
+        s2r = torch.empty(n * top_k, dtype=torch.int64, device=dev)
+        ws = _workspace(lib.fmoe_routing_workspace_bytes(n * top_k, e), dev)
+        check(lib.fmoe_noisy_gate_forward(_ptr(clean), _ptr(raw), _ptr(noise), float(eps), n, e, top_k, dt, _ptr(idx),
+                                          _ptr(gates), _ptr(thr_val), _ptr(thr_idx), _ptr(partial), _ptr(cnt), _ptr(pos),
+                                          _ptr(s2r), _ptr(ws), ws.numel(), _stream(clean)))
+        load = partial.sum(dim=0)
+    return idx, gates, load, thr_val, thr_idx, cnt, pos, s2r
+
+
+def noisy_gate_backward(clean, raw, noise, top_k, eps, topk_idx, gates, thr_val, thr_idx, grad_gates, grad_load):
+    """Gradients of ``clean`` and ``raw`` ``[N, E]`` from those of the gates ``[N, k]`` and the load ``[E]``."""
+    dt = _rows("clean", clean)
+    _dev("grad_gates", grad_gates, clean.dtype)
+    _dev("grad_load", grad_load, torch.float32)
+    n, e = clean.shape
+    grad_clean, grad_raw = torch.empty_like(clean), torch.empty_like(clean)
+    with torch.cuda.device(clean.device):
+        check(_lib.load().fmoe_noisy_gate_backward(_ptr(clean), _ptr(raw), _ptr(noise), float(eps), n, e, top_k, dt,
+                                                   _ptr(topk_idx), _ptr(gates), _ptr(thr_val), _ptr(thr_idx),
+                                                   _ptr(grad_gates), _ptr(grad_load), _ptr(grad_clean), _ptr(grad_raw),
+                                                   _stream(clean)))
+    return grad_clean, grad_raw
+
+
 def gate_topk_backward(grad_score, score, topk_idx, n_expert, score_mode=0):
     """Gradient of the top-k scores with respect to the logits, ``[N, E]``."""
     _dev("grad_score", grad_score)

@@ -89,6 +89,36 @@ def gate_linear_topk(x, linear, top_k, score_mode=0):
     return gate_topk(linear(x), top_k, score_mode)
 
 
+class NoisyTopK(Function):
+    r"""The training-mode selection of the noisy top-k gate (fmoe/gates/noisy_gate.py:113-144) after
+    its two linear products: ``(topk_idx [N,k], gates [N,k], load [E])`` from the clean logits, the raw
+    noise widths and a draw of N(0,1) noise, with the routing of ``count_by_gate`` riding on ``topk_idx``.
+    ``load`` is the smooth estimate of tokens per expert (float32); both ``gates`` and ``load`` are
+    differentiable with respect to ``clean`` and ``raw``."""
+
+    @staticmethod
+    def forward(ctx, clean, raw, noise, top_k, eps):
+        clean, raw, noise = clean.contiguous(), raw.contiguous(), noise.contiguous()
+        idx, gates, load, thr_val, thr_idx, cnt, pos_buf, s2r = fmoe_native.noisy_gate_forward(clean, raw, noise, top_k, eps)
+        ctx.save_for_backward(clean, raw, noise, idx, gates, thr_val, thr_idx)
+        ctx.moe_args = top_k, eps
+        ctx.mark_non_differentiable(idx)
+        idx._fmoe_route = (idx._version, clean.shape[1], cnt, pos_buf, s2r)
+        return idx, gates, load
+
+    @staticmethod
+    def backward(ctx, _grad_idx, grad_gates, grad_load):
+        clean, raw, noise, idx, gates, thr_val, thr_idx = ctx.saved_tensors
+        top_k, eps = ctx.moe_args
+        if grad_gates is None:
+            grad_gates = torch.zeros_like(gates)
+        if grad_load is None:
+            grad_load = torch.zeros(clean.shape[1], dtype=torch.float32, device=clean.device)
+        g_clean, g_raw = fmoe_native.noisy_gate_backward(clean, raw, noise, top_k, eps, idx, gates, thr_val, thr_idx,
+                                                         grad_gates.contiguous(), grad_load.float().contiguous())
+        return g_clean, g_raw, None, None, None
+
+
 def gate_topk(logits, top_k, score_mode=0):
     r"""Top-k indices and scores of ``logits [N, E]``: the HIP gate kernel when it takes the shape
     (CUDA tensor, 16/32-bit floats, ``top_k`` 1, 2, 4 or 8), ``torch.topk``

@@ -144,6 +144,43 @@ int fmoe_gate_topk_backward(const void *grad_score, const void *score,
                             int64_t n_tokens, int64_t n_expert, int64_t top_k,
                             int dtype, int score_mode, void *stream);
 
+/* Noisy top-k gating in training mode (Shazeer et al. 2017; the behaviour of
+ * fmoe/gates/noisy_gate.py:113-144) after the two linear products, in one
+ * pass: with std = softplus(raw) + eps and noisy = clean + noise * std (clean,
+ * raw, noise [n_tokens, n_expert] of `dtype`; noise is the caller's N(0,1)
+ * draw), per token the top_k + 1 largest noisy logits,
+ *   topk_idx [n_tokens, top_k] int64, gates [n_tokens, top_k] = softmax over
+ *   the top_k largest;  thr_val / thr_idx [n_tokens, 2]: the top_k-th and
+ *   (top_k+1)-th largest noisy logit and their experts (kept for the backward);
+ *   load_partial [ceil(n_tokens*top_k / 2048), n_expert] float: per workgroup
+ *   the sums over its tokens of Phi((clean - threshold) / std), threshold =
+ *   the (top_k+1)-th largest noisy logit for an expert among the top_k, the
+ *   top_k-th otherwise; the load is the sum of the rows;
+ * and expert_count / pos / slot_to_row as fmoe_route(topk_idx) gives them.
+ * top_k 1, 2, 4 or 8 and below n_expert <= 2048 (FMOE_ELIMIT otherwise).
+ * workspace: fmoe_routing_workspace_bytes(n_tokens*top_k, n_expert). */
+int fmoe_noisy_gate_forward(const void *clean, const void *raw,
+                            const void *noise, double eps, int64_t n_tokens,
+                            int64_t n_expert, int64_t top_k, int dtype,
+                            int64_t *topk_idx, void *gates, float *thr_val,
+                            int32_t *thr_idx, float *load_partial,
+                            int64_t *expert_count, int64_t *pos,
+                            int64_t *slot_to_row, void *workspace,
+                            int64_t workspace_bytes, void *stream);
+
+/* Its backward: from grad_gates [n_tokens, top_k] (`dtype`) and grad_load
+ * [n_expert] (float), the gradients of the two logit matrices, grad_clean and
+ * grad_raw [n_tokens, n_expert] (`dtype`), through the softmax, the smooth load
+ * (including its thresholds) and the softplus.  Replaces autograd's backward of
+ * fmoe/gates/noisy_gate.py:47-90,113-144. */
+int fmoe_noisy_gate_backward(const void *clean, const void *raw,
+                             const void *noise, double eps, int64_t n_tokens,
+                             int64_t n_expert, int64_t top_k, int dtype,
+                             const int64_t *topk_idx, const void *gates,
+                             const float *thr_val, const int32_t *thr_idx,
+                             const void *grad_gates, const float *grad_load,
+                             void *grad_clean, void *grad_raw, void *stream);
+
 /* ---- capacity balancing ------------------------------------------------- */
 
 /* eca[w,e] = share of cap[e] granted to worker w, workers served in ascending

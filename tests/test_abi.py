@@ -48,6 +48,8 @@ def test_ctypes_signatures_match_the_header():
                 assert a is ctypes.c_void_p or issubclass(a, ctypes._Pointer), f"{name}: `{q}` is a pointer"
             elif q.startswith("int64_t"):
                 assert a is ctypes.c_int64, f"{name}: `{q}` is int64_t"
+            elif q.startswith("double"):
+                assert a is ctypes.c_double, f"{name}: `{q}` is double"
             else:
                 assert q.startswith("int ") and a is ctypes.c_int, f"{name}: `{q}`"
         if "*" in ret:

@@ -46,6 +46,9 @@ def _compare(moe, x, act, top_k, dtype, grads_of_score=False):
             assert ref[name] is None
             continue
         assert rel_err(val, ref[name]) <= tol, (name, rel_err(val, ref[name]))
+        if dtype == torch.float32:
+            # float32 is held to the element-by-element and root-mean-square bounds as well
+            assert_close(val, ref[name], tol, name)
     return got
 
 
@@ -777,8 +780,9 @@ def test_bf16_configurations_at_full_size_sampled_against_the_oracle(name, n, d,
     sample = torch.randperm(n, generator=torch.Generator().manual_seed(5))[:48].to(device)
     ref = omoe.moe_mlp_forward_backward_per_expert(x[sample], idx[sample], score[sample], w1, b1, w2, b2, "gelu", k,
                                                    grad_out=grad[sample], grad_dtype=torch.float32)
-    assert_close(out[sample], ref["out"], 2e-2, f"{name}: output of the sampled tokens", floor=3.0)
-    assert_close(x.grad[sample], ref["grad_inp"], 2e-2, f"{name}: input gradient of the sampled tokens", floor=3.0)
+    # (two roundings to bfloat16 on the way to these: floor 1; the weight gradients below, four and a long sum: 3)
+    assert_close(out[sample], ref["out"], 2e-2, f"{name}: output of the sampled tokens", floor=1.0)
+    assert_close(x.grad[sample], ref["grad_inp"], 2e-2, f"{name}: input gradient of the sampled tokens", floor=1.0)
     del ref
 
     # -- the largest expert, 8 hidden units: weight and bias gradients over all of the expert's rows
@@ -960,3 +964,73 @@ def test_layer_forward_in_a_hip_graph_with_new_routing_per_replay(dtype, device)
             torch.cuda.synchronize()
             assert torch.equal(got, want), f"replay {rep}"
     assert len(counts_seen) >= 3   # the replays really routed differently
+
+
+@pytest.mark.parametrize("dtype", [torch.float32])
+@pytest.mark.parametrize("n,d,e,k", [(40, 16, 6, 2), (3000, 64, 64, 4), (1111, 32, 300, 8), (700, 48, 9, 1)])
+def test_noisy_gate_kernel_against_the_torch_formulation(dtype, n, d, e, k, device, monkeypatch):
+    """NoisyGate in training mode: the one-pass kernel (noise, softplus, top-(k+1), softmax, smooth load,
+    routing) and its backward against the same gate written out in torch operators
+    (FMOE_NOISY_GATE_KERNEL=0) with the same noise draw: indices, gates, loss, and the gradients of
+    both weight matrices and of the input through loss + gates; the routing against the oracle."""
+    torch.manual_seed(n + e)
+    gate = NoisyGate(d, e, 1, top_k=k).to(device)
+    with torch.no_grad():
+        gate.w_gate.normal_(0, 1.0 / d ** 0.5)
+        gate.w_noise.normal_(0, 1.0 / d ** 0.5)
+    gate = gate.to(dtype)
+    gate.train()
+    x = torch.randn(n, d, device=device).to(dtype)
+    g = torch.randn(n, 1, k, device=device).to(dtype)
+    results = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("FMOE_NOISY_GATE_KERNEL", flag)
+        gate.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        torch.manual_seed(5)
+        idx, score = gate(xi)
+        loss = gate.get_loss()
+        (loss + (score * g).float().sum()).backward()
+        results.append((idx, score, loss.detach(), xi.grad, gate.w_gate.grad.clone(), gate.w_noise.grad.clone()))
+        if flag == "1":
+            assert hasattr(idx, "_fmoe_route")
+            cnt, pos_buf, s2r = idx._fmoe_route[2:]
+            ref_pos, ref_cnt = orouting.count_by_gate(idx.cpu().numpy(), e)
+            assert np.array_equal(cnt.cpu().numpy(), ref_cnt) and np.array_equal(pos_buf.cpu().numpy(), ref_pos)
+    (idx_a, sc_a, loss_a, gx_a, gwg_a, gwn_a), (idx_b, sc_b, loss_b, gx_b, gwg_b, gwn_b) = results
+    assert torch.equal(idx_a, idx_b)
+    assert torch.allclose(sc_a, sc_b, rtol=1e-5, atol=1e-6)
+    assert abs(float(loss_a) - float(loss_b)) <= 1e-4 * abs(float(loss_b))
+    for a, b in ((gx_a, gx_b), (gwg_a, gwg_b), (gwn_a, gwn_b)):
+        assert rel_err(a, b) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,e,k", [(3000, 64, 4), (500, 12, 2)])
+def test_noisy_top_k_16_bit_against_float64(dtype, n, e, k, device):
+    """NoisyTopK on 16-bit logits (the kernel computes in float32 and rounds its outputs once) against
+    the same formulas in float64 on the same 16-bit inputs: indices equal, gates / load / gradients
+    within 2e-2."""
+    from fastermoe_amd.functions import NoisyTopK
+    torch.manual_seed(e)
+    clean = torch.randn(n, e, device=device).to(dtype).requires_grad_(True)
+    raw = torch.randn(n, e, device=device).to(dtype).requires_grad_(True)
+    noise = torch.randn(n, e, device=device).to(dtype)
+    gg = torch.randn(n, k, device=device).to(dtype)
+    gl = torch.randn(e, device=device)
+    idx, gates, load = NoisyTopK.apply(clean, raw, noise, k, 1e-2)
+    ((gates * gg).float().sum() + (load * gl).sum()).backward()
+    c64, r64 = clean.detach().double().requires_grad_(True), raw.detach().double().requires_grad_(True)
+    std = torch.nn.functional.softplus(r64) + 1e-2
+    noisy = c64 + noise.double() * std
+    top_vals, top_idx = noisy.topk(k + 1, dim=1)
+    assert torch.equal(idx, top_idx[:, :k])
+    ref_gates = torch.softmax(top_vals[:, :k], dim=1)
+    inside = noisy > top_vals[:, k:k + 1]
+    thr = torch.where(inside, top_vals[:, k:k + 1], top_vals[:, k - 1:k])
+    ref_load = torch.special.ndtr((c64 - thr) / std).sum(dim=0)
+    ((ref_gates * gg.double()).sum() + (ref_load * gl.double()).sum()).backward()
+    tol = TOL[dtype]
+    assert rel_err(gates, ref_gates) <= tol and rel_err(load, ref_load) <= 1e-4
+    assert_close(clean.grad, c64.grad, tol, "grad_clean")
+    assert_close(raw.grad, r64.grad, tol, "grad_raw")

@@ -69,3 +69,36 @@ def test_route_static_rejects_sizes_beyond_its_array(device):
     rc = lib.fmoe_route_static(_vp(dummy), n, e, _vp(cnt), _vp(dummy), None, None)
     assert rc == -2  # FMOE_ELIMIT
     assert b"fmoe_route_static" in lib.fmoe_last_error()
+
+
+def test_route_static_allocates_no_device_memory(device):
+    """Free device memory, as the driver reports it, is the same before and after calls of
+    fmoe_route_static on buffers that exist already -- and the call can be captured into a HIP graph,
+    which an allocating call could not be."""
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(3)
+    n, k, e = 4096, 2, 32
+    gate = torch.randint(-1, e, (n, k), generator=gen).to(device)
+    cnt = torch.empty(e, dtype=torch.int64, device=device)
+    pos = torch.empty(n * k, dtype=torch.int64, device=device)
+    s2r = torch.empty(n * k, dtype=torch.int64, device=device)
+    st = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    _lib.check(lib.fmoe_route_static(_vp(gate), n * k, e, _vp(cnt), _vp(pos), _vp(s2r), st))   # first call: symbol lookup
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(device)
+    for _ in range(5):
+        _lib.check(lib.fmoe_route_static(_vp(gate), n * k, e, _vp(cnt), _vp(pos), _vp(s2r), st))
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(device)
+    assert free_after == free_before
+    want = (cnt.clone(), pos.clone(), s2r.clone())
+    # under capture (no allocation is allowed there), replayed on another gate tensor's contents
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cap = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+        _lib.check(lib.fmoe_route_static(_vp(gate), n * k, e, _vp(cnt), _vp(pos), _vp(s2r), cap))
+    for rep in range(3):
+        cnt.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(cnt, want[0]) and torch.equal(pos, want[1]) and torch.equal(s2r, want[2]), rep
