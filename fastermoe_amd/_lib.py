@@ -58,8 +58,10 @@ SIGNATURES = {
     "fmoe_segment_table_bytes": (_i64, [_i64, _i64]),
     "fmoe_segment_table_build": (_int, [_vp, _i64, _i64, _vp, _i64, _vp]),
     "fmoe_linear_dev_supported": (_int, [_i64, _i64, _int]),
-    "fmoe_linear_forward_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
-    "fmoe_linear_dgrad_dev": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "fmoe_linear_dev_workspace_bytes": (_i64, [_i64, _int]),
+    "fmoe_linear_forward_dev": (_int, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp,
+                                       _i64, _vp]),
+    "fmoe_linear_dgrad_dev": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _i64, _vp]),
     "fmoe_linear_wgrad_dev": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "fmoe_gemm_tail_plan": (_int, [_i64, _i64, _int, _vp]),
     "fmoe_fused_chunk_bounds": (_int, [_vp, _i64, _int, _i64, _i64, _int, _vp]),

@@ -204,6 +204,11 @@ struct GemmParams {
     // the expert count (any number), tab.first_expert 0, and nothing is split.
     const int32_t *dev_tab;
     int32_t dev_map_off;       // offset (in int32) of the tile map for this launch's tile height
+    // Device table and a caller's workspace for split tail tiles: dev_cus > 0 makes every workgroup plan
+    // the tail split itself from the table's tile count, for dev_cus compute units (host only: dev_split_ws,
+    // the workspace of at least dev_cus tiles of fp32 accumulators, copied to split_ws for the launch)
+    int32_t dev_cus;
+    float *dev_split_ws;
     int64_t dev_rows_cap;      // host only: rows the device table was laid out for
     int32_t block_m, block_n;  // host only: tile height the segment table was built for (256 or 128) and tile width
     int32_t profile_class;     // host only: ProfileClass of this launch
@@ -222,6 +227,38 @@ inline void set_row_index_divisor(GemmParams &prm, int64_t divisor) {
     while (((int64_t)1 << s) < divisor) ++s;
     prm.q_div_mul = (uint32_t)((((uint64_t)1 << (31 + s)) / (uint64_t)divisor) + 1);
     prm.q_div_shift = s - 1;   // after the multiply-high's shift by 32
+}
+
+// How the tiles of a ragged-rows launch are spread over the chip.  One workgroup occupies a
+// compute unit, so `total` tiles run in total / cus rounds and a last, partial round costs as
+// much as a whole one.  When that last round fills at most half the chip, its tiles are split
+// along the contraction into k_split parts (as many as fit the idle units, at most 8, at
+// least 16 slabs each) -- provided that shortens the round by more than the partial sums' round
+// trip through memory costs.  Evaluated on the host for launches over host counts and by every
+// workgroup for launches over a device table (where only the device knows the tile count).
+constexpr int kMaxSplit = 8;
+struct TailSplit {
+    int main_tiles, k_split, split_slabs;
+};
+__host__ __device__ inline TailSplit plan_tail_split(int total, int n_slabs, int cus) {
+    TailSplit p{total, 1, n_slabs};
+    const int tail = total % cus;
+    if (tail == 0 || tail * 2 > cus) return p;
+    int f = cus / tail < kMaxSplit ? cus / tail : kMaxSplit;
+    f = n_slabs / 16 < f ? n_slabs / 16 : f;
+    if (f < 2) return p;
+    const int per_part = (n_slabs + f - 1) / f;
+    // the reduction and the second launch cost about as much as 40 slabs of one tile
+    if (n_slabs - per_part < 40) return p;
+    p.split_slabs = per_part;
+    p.k_split = (n_slabs + p.split_slabs - 1) / p.split_slabs;  // no empty part
+    p.main_tiles = total - tail;
+    return p;
+}
+// whether any tile count at all makes plan_tail_split split a contraction of n_slabs slabs
+inline bool tail_split_possible(int n_slabs) {
+    const int f = n_slabs / 16 < kMaxSplit ? n_slabs / 16 : kMaxSplit;
+    return f >= 2 && n_slabs - (n_slabs + f - 1) / f >= 40;
 }
 
 // KC slabs: 16-byte chunk c of row r is stored at chunk c ^ swz(r).
@@ -264,6 +301,7 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
     int split_part = -1;   // >= 0: this workgroup computes that part of the contraction of a tail tile
     int tail_index = 0;    // index of a tail tile among the tail tiles
     const bool fixup = RAGGED == kRaggedRows && prm.fixup != 0;
+    int k_split = prm.k_split, split_slabs = prm.split_slabs;  // (a launch over a device table plans them below)
     // the device table is read-only while the kernel runs and addressed uniformly: scalar loads
     typedef const int32_t __attribute__((address_space(4))) *DevTab;
     const DevTab dtab = (DevTab)(uintptr_t)prm.dev_tab;
@@ -277,20 +315,28 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
             if (dev) {
                 tm_total = dtab[BM == 256 ? segtab::kTiles256 : segtab::kTiles128];
                 main_tiles = total_tiles = tm_total * prm.tiles_n;
+                if (prm.dev_cus > 0) {
+                    const TailSplit ts = plan_tail_split(total_tiles, (prm.k_extent + BKE - 1) / BKE, prm.dev_cus);
+                    main_tiles = ts.main_tiles;
+                    k_split = ts.k_split;
+                    split_slabs = ts.split_slabs;
+                }
             } else {
                 tm_total = prm.tab.tile[prm.tab.n];
             }
             const int main_grid = (main_tiles + 7) & ~7;
             if (fixup) {
                 tail_index = blockIdx.x / kWaves;  // one one-wave workgroup per wave of a tail tile
+                // (device table: the launch was sized for the most tail tiles there can be)
+                if (dev && (k_split == 1 || tail_index >= total_tiles - main_tiles)) return;
                 L = main_tiles + tail_index;
             } else if ((int)blockIdx.x < main_grid) {
                 const int per_xcd = main_grid >> 3;
                 L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
                 if (L >= main_tiles) return;
             } else {
-                if (dev) return;  // the launch was sized for an upper bound of tiles
                 const int u = blockIdx.x - main_grid, n_tail = total_tiles - main_tiles;
+                if (dev && (k_split == 1 || u >= n_tail * k_split)) return;  // the launch was sized for an upper bound
                 split_part = u / n_tail;
                 tail_index = u - split_part * n_tail;
                 L = main_tiles + tail_index;
@@ -362,8 +408,8 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
         Pb = (PSHAPE == kKC) ? Pe + (int64_t)n0 * prm.ldp : Pe + n0;
         aux_off = (int64_t)row0 * prm.ldc + n0;
         if (split_part >= 0) {  // this part's slabs only
-            const int k_begin = split_part * prm.split_slabs * BKE;
-            K = max(0, min(K - k_begin, prm.split_slabs * BKE));
+            const int k_begin = split_part * split_slabs * BKE;
+            K = max(0, min(K - k_begin, split_slabs * BKE));
             Qb += (QSHAPE == kKC) ? (int64_t)k_begin : (int64_t)k_begin * prm.ldq;
             q_gather_bytes = -(int64_t)k_begin * (int64_t)sizeof(T);
             Pb += (PSHAPE == kKC) ? (int64_t)k_begin : (int64_t)k_begin * prm.ldp;
@@ -810,7 +856,7 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
         constexpr int kVecPerBlk = kAccRegs / 4;
         constexpr int64_t kTileVecs = (int64_t)BM * BN / 4;
         if (split_part >= 0) {
-            f32x4 *dst = (f32x4 *)prm.split_ws + ((int64_t)tail_index * prm.k_split + split_part) * kTileVecs + t;
+            f32x4 *dst = (f32x4 *)prm.split_ws + ((int64_t)tail_index * k_split + split_part) * kTileVecs + t;
 #pragma unroll
             for (int x = 0; x < TI; ++x)
 #pragma unroll
@@ -827,7 +873,7 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
         }
         if (fixup) {
             // the parts have been added up into part 0 by split_reduce_kernel; loads go out eight at a time
-            const f32x4 *src = (const f32x4 *)prm.split_ws + (int64_t)tail_index * prm.k_split * kTileVecs + wave * 64 + lane;
+            const f32x4 *src = (const f32x4 *)prm.split_ws + (int64_t)tail_index * k_split * kTileVecs + wave * 64 + lane;
             constexpr int kVecs = TI * TJ * kVecPerBlk, kBatch = 8;
             static_assert(kVecs % kBatch == 0, "accumulator vectors are loaded in batches of eight");
 #pragma unroll
@@ -1084,37 +1130,35 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(float *ws, int k_spli
         if (p < k_split) sum += part[p];
     base[0] = sum;
 }
-constexpr int kMaxSplit = 8;
+
+// The same for a launch over a device table: sized for the most tail tiles there can be, every
+// thread works out from the table's tile count whether (and how) the tail was split.
+template <int kMaxSplit>
+__global__ __launch_bounds__(256) void split_reduce_dev_kernel(float *ws, const int32_t *__restrict__ dev_tab, int tiles_index,
+                                                               int tiles_n, int n_slabs, int cus, int64_t tile_vecs) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int total = dev_tab[tiles_index] * tiles_n;
+    const TailSplit ts = plan_tail_split(total, n_slabs, cus);
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t tile = i / tile_vecs, v = i - tile * tile_vecs;
+    if (ts.k_split == 1 || tile >= total - ts.main_tiles) return;
+    f32x4 *base = (f32x4 *)ws + tile * ts.k_split * tile_vecs + v;
+    f32x4 part[kMaxSplit];
+#pragma unroll
+    for (int p = 0; p < kMaxSplit; ++p)
+        if (p < ts.k_split) part[p] = __builtin_nontemporal_load(base + (int64_t)p * tile_vecs);
+    f32x4 sum = part[0];
+#pragma unroll
+    for (int p = 1; p < kMaxSplit; ++p)
+        if (p < ts.k_split) sum += part[p];
+    base[0] = sum;
+}
 
 // Host-side services of grouped_gemm.hip: compute units of the current device, and a per-stream
 // buffer for the partial accumulators of split tail tiles (allocated on first use, kept until
 // the process ends; NULL when the allocation fails, in which case nothing is split).
 int device_compute_units();
 float *split_workspace(hipStream_t stream, size_t bytes);
-
-// How the tiles of a ragged-rows launch are spread over the chip.  One workgroup occupies a
-// compute unit, so `total` tiles run in total / cus rounds and a last, partial round costs as
-// much as a whole one.  When that last round fills at most half the chip, its tiles are split
-// along the contraction into k_split parts (as many as fit the idle units, at most 8, at
-// least 16 slabs each) -- provided that shortens the round by more than the partial sums' round
-// trip through memory costs.
-struct TailSplit {
-    int main_tiles, k_split, split_slabs;
-};
-inline TailSplit plan_tail_split(int total, int n_slabs, int cus) {
-    TailSplit p{total, 1, n_slabs};
-    const int tail = total % cus;
-    if (tail == 0 || tail * 2 > cus) return p;
-    int f = std::min(std::min(kMaxSplit, cus / tail), n_slabs / 16);
-    if (f < 2) return p;
-    const int per_part = (n_slabs + f - 1) / f;
-    // the reduction and the second launch cost about as much as 40 slabs of one tile
-    if (n_slabs - per_part < 40) return p;
-    p.split_slabs = per_part;
-    p.k_split = (n_slabs + p.split_slabs - 1) / p.split_slabs;  // no empty part
-    p.main_tiles = total - tail;
-    return p;
-}
 
 template <typename T, int BM, int BN, int PS, int QS, int RG, int EPI>
 int launch_tiles(GemmParams &prm, hipStream_t stream) {
@@ -1149,22 +1193,31 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
         constexpr int BKE = kSlabBytes / (int)sizeof(T);
         const int n_slabs = (prm.k_extent + BKE - 1) / BKE;
         // (two 128 x 128 workgroups share a compute unit: their launches are not split)
-        // (nor is a launch over a device table, whose tile count the host does not know)
-        const TailSplit ts = (BN == 256 && prm.dev_tab == nullptr)
-                                 ? plan_tail_split(prm.total_tiles, n_slabs, device_compute_units())
-                                 : TailSplit{prm.total_tiles, 1, n_slabs};
-        if (ts.k_split > 1) {
-            const int tail = prm.total_tiles - ts.main_tiles;
-            float *ws = split_workspace(stream, (size_t)tail * ts.k_split * BM * BN * sizeof(float));
-            if (ws != nullptr) {
-                prm.split_ws = ws;
-                prm.main_tiles = ts.main_tiles;
-                prm.k_split = ts.k_split;
-                prm.split_slabs = ts.split_slabs;
+        if (prm.dev_tab != nullptr) {
+            // the host does not know the tile count: with a workspace from the caller, every workgroup plans the
+            // split itself, and the launch is sized for the most parts there can be (one per compute unit)
+            prm.dev_cus = 0;
+            if (BN == 256 && prm.dev_split_ws != nullptr && tail_split_possible(n_slabs)) {
+                prm.dev_cus = device_compute_units();
+                prm.split_ws = prm.dev_split_ws;
             }
+            grid64 = ((int64_t)prm.total_tiles + 7) / 8 * 8 + prm.dev_cus;
+        } else {
+            const TailSplit ts = BN == 256 ? plan_tail_split(prm.total_tiles, n_slabs, device_compute_units())
+                                           : TailSplit{prm.total_tiles, 1, n_slabs};
+            if (ts.k_split > 1) {
+                const int tail = prm.total_tiles - ts.main_tiles;
+                float *ws = split_workspace(stream, (size_t)tail * ts.k_split * BM * BN * sizeof(float));
+                if (ws != nullptr) {
+                    prm.split_ws = ws;
+                    prm.main_tiles = ts.main_tiles;
+                    prm.k_split = ts.k_split;
+                    prm.split_slabs = ts.split_slabs;
+                }
+            }
+            // whole tiles rounded up to a multiple of 8 (one range per XCD), then the parts of the tail tiles
+            grid64 = ((int64_t)prm.main_tiles + 7) / 8 * 8 + (int64_t)(prm.total_tiles - prm.main_tiles) * prm.k_split;
         }
-        // whole tiles rounded up to a multiple of 8 (one range per XCD), then the parts of the tail tiles
-        grid64 = ((int64_t)prm.main_tiles + 7) / 8 * 8 + (int64_t)(prm.total_tiles - prm.main_tiles) * prm.k_split;
     } else {
         // 8 XCDs x experts x an eighth (rounded up) of one expert's tiles -- the kernel drops the surplus workgroups
         grid64 = (int64_t)8 * prm.tab.n * (((int64_t)prm.tiles_m * prm.tiles_n + 7) / 8);
@@ -1183,6 +1236,19 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
         FMOE_LAUNCH_CHECK();
         prm.fixup = 1;
         kern<<<(prm.total_tiles - prm.main_tiles) * kWavesM * kWavesN, 64, smem_wave_epi, stream>>>(prm);
+        FMOE_LAUNCH_CHECK();
+        prm.fixup = 0;
+    } else if (RG == kRaggedRows && prm.dev_tab != nullptr && prm.dev_cus > 0) {
+        // device table: the same two steps, sized for the most tail tiles a split can have (half the chip)
+        constexpr int BKE = kSlabBytes / (int)sizeof(T);
+        const int max_tail = prm.dev_cus / 2;
+        const int64_t tile_vecs = (int64_t)BM * BN / 4;
+        split_reduce_dev_kernel<kMaxSplit><<<(unsigned)((tile_vecs * max_tail + 255) / 256), 256, 0, stream>>>(
+            prm.split_ws, prm.dev_tab, BM == 256 ? segtab::kTiles256 : segtab::kTiles128, prm.tiles_n,
+            (prm.k_extent + BKE - 1) / BKE, prm.dev_cus, tile_vecs);
+        FMOE_LAUNCH_CHECK();
+        prm.fixup = 1;
+        kern<<<max_tail * kWavesM * kWavesN, 64, smem_wave_epi, stream>>>(prm);
         FMOE_LAUNCH_CHECK();
         prm.fixup = 0;
     }

@@ -370,6 +370,15 @@ int device_table_launch(const char *who, GemmParams &prm, const int32_t *dev_tab
     return FMOE_OK;
 }
 
+int64_t linear_dev_workspace_bytes(int64_t contraction, int dtype) {
+    const int eb = dtype_bytes(dtype);
+    if (eb == 0 || dtype == FMOE_F64 || contraction < 1) return 0;
+    const int64_t per_slab = kSlabBytes / eb;
+    if (!tail_split_possible((int)std::min<int64_t>(ceil_div(contraction, per_slab), 1 << 24))) return 0;
+    // one tile of fp32 accumulators per compute unit: a split never has more parts than that
+    return (int64_t)device_compute_units() * 256 * 256 * (int64_t)sizeof(float);
+}
+
 int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, int64_t n_expert, int64_t row_lo,
                            int64_t row_hi, hipStream_t stream) {
     if (a.dev_tab != nullptr) {
@@ -392,6 +401,9 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
         prm.bias_expert_stride = a.out_feat;
         prm.n_cols = (int)a.out_feat; prm.k_extent = (int)a.in_feat;
         prm.activation = a.activation;
+        const int64_t ws_need = linear_dev_workspace_bytes(a.in_feat, a.dtype);
+        if (a.dev_workspace != nullptr && ws_need > 0 && a.dev_workspace_bytes >= ws_need && aligned16(a.dev_workspace))
+            prm.dev_split_ws = (float *)a.dev_workspace;
         return dispatch<kFwd>(prm, a.dtype, a.epilogue, fast, stream);
     }
     int64_t total;
@@ -441,6 +453,9 @@ int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts, int64_
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.n_cols = (int)a.in_feat; prm.k_extent = (int)a.out_feat;
         prm.activation = a.activation;
+        const int64_t ws_need = linear_dev_workspace_bytes(a.out_feat, a.dtype);
+        if (a.dev_workspace != nullptr && ws_need > 0 && a.dev_workspace_bytes >= ws_need && aligned16(a.dev_workspace))
+            prm.dev_split_ws = (float *)a.dev_workspace;
         return dispatch<kDgrad>(prm, a.dtype, a.epilogue, fast, stream);
     }
     int64_t total;
@@ -623,10 +638,15 @@ extern "C" int fmoe_linear_dev_supported(int64_t in_feat, int64_t out_feat, int 
     return (in_feat % ce == 0 && out_feat % ce == 0 && in_feat * eb <= (1 << 22) && out_feat * eb <= (1 << 22)) ? 1 : 0;
 }
 
+extern "C" int64_t fmoe_linear_dev_workspace_bytes(int64_t contraction, int dtype) {
+    return linear_dev_workspace_bytes(contraction, dtype);
+}
+
 extern "C" int fmoe_linear_forward_dev(const void *x, const int64_t *x_row_index, int64_t x_index_div,
                                        int64_t x_total_rows, const void *w, const void *bias, void *pre, void *y,
                                        const void *segment_table, int64_t n_expert, int64_t rows_cap, int64_t in_feat,
-                                       int64_t out_feat, int dtype, int activation, void *stream) {
+                                       int64_t out_feat, int dtype, int activation, void *workspace,
+                                       int64_t workspace_bytes, void *stream) {
     FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_forward_dev: unknown dtype %d", dtype);
     FMOE_REQUIRE(activation >= FMOE_ACT_NONE && activation <= FMOE_ACT_GELU, "fmoe_linear_forward_dev: activation %d",
                  activation);
@@ -640,12 +660,15 @@ extern "C" int fmoe_linear_forward_dev(const void *x, const int64_t *x_row_index
     a.x_total_rows = x_row_index ? x_total_rows : 0;
     a.dev_tab = (const int32_t *)segment_table;
     a.dev_rows_cap = rows_cap;
+    a.dev_workspace = workspace;
+    a.dev_workspace_bytes = workspace_bytes;
     return grouped_linear_forward(a, nullptr, n_expert, 0, rows_cap, (hipStream_t)stream);
 }
 
 extern "C" int fmoe_linear_dgrad_dev(const void *grad_y, const void *w, const void *pre, void *grad_x,
                                      const void *segment_table, int64_t n_expert, int64_t rows_cap, int64_t in_feat,
-                                     int64_t out_feat, int dtype, int activation, void *stream) {
+                                     int64_t out_feat, int dtype, int activation, void *workspace,
+                                     int64_t workspace_bytes, void *stream) {
     FMOE_REQUIRE(dtype_bytes(dtype) != 0, "fmoe_linear_dgrad_dev: unknown dtype %d", dtype);
     FMOE_REQUIRE(activation >= FMOE_ACT_NONE && activation <= FMOE_ACT_GELU, "fmoe_linear_dgrad_dev: activation %d",
                  activation);
@@ -656,6 +679,8 @@ extern "C" int fmoe_linear_dgrad_dev(const void *grad_y, const void *w, const vo
                       has_act ? kEpiDAct : kEpiStore, activation};
     d.dev_tab = (const int32_t *)segment_table;
     d.dev_rows_cap = rows_cap;
+    d.dev_workspace = workspace;
+    d.dev_workspace_bytes = workspace_bytes;
     return grouped_linear_dgrad(d, nullptr, n_expert, 0, rows_cap, (hipStream_t)stream);
 }
 

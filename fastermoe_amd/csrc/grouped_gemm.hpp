@@ -69,7 +69,15 @@ struct LinearForwardArgs {
     // host counts are then not read (may be NULL) and the row range must be everything
     const int32_t *dev_tab = nullptr;
     int64_t dev_rows_cap = 0;
+    // optional, with dev_tab: workspace of linear_dev_workspace_bytes() for the split of a last, partial
+    // round of tiles (without it such a round is not split)
+    void *dev_workspace = nullptr;
+    int64_t dev_workspace_bytes = 0;
 };
+
+// Bytes of workspace with which a launch over a device table can split its last round of tiles along a
+// contraction of `contraction` elements; 0 when a contraction this short is never split.
+int64_t linear_dev_workspace_bytes(int64_t contraction, int dtype);
 
 // Whether the forward product can read its rows through an index: the MFMA path (aligned pointers,
 // feature sizes that are multiples of 16 bytes) and a token matrix of less than 2 GiB.
@@ -84,6 +92,8 @@ struct LinearDgradArgs {
     int dtype, epilogue, activation;
     const int32_t *dev_tab = nullptr;  // as in LinearForwardArgs
     int64_t dev_rows_cap = 0;
+    void *dev_workspace = nullptr;
+    int64_t dev_workspace_bytes = 0;
 };
 
 struct LinearWgradArgs {

@@ -584,6 +584,16 @@ def linear_dev_supported(in_feat, out_feat, dtype):
     return dtype in _DTYPES and _lib.load().fmoe_linear_dev_supported(int(in_feat), int(out_feat), _DTYPES[dtype]) == 1
 
 
+def _dev_workspace(contraction, dt, device):
+    """The caller-side workspace of the row-ragged ``*_dev`` products (``None`` when this contraction is
+    never split); torch's caching allocator hands the same block back call after call."""
+    import os
+    nbytes = _lib.load().fmoe_linear_dev_workspace_bytes(int(contraction), dt)
+    if nbytes == 0 or os.environ.get("FMOE_DEV_SPLIT", "1") == "0":
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
 def _check_table(table, n_expert, rows_cap):
     _dev("segment_table", table, torch.int32)
     need = _lib.load().fmoe_segment_table_bytes(int(rows_cap), int(n_expert)) // 4
@@ -617,9 +627,11 @@ def linear_forward_dev(x, weight, bias, table, rows_cap, activation=_lib.ACT_NON
     y = new()
     pre = new() if keep_pre else None
     with torch.cuda.device(x.device):
+        ws = _dev_workspace(in_feat, dt, x.device)
         check(_lib.load().fmoe_linear_forward_dev(_ptr(x), _ptr(row_index), int(index_div), x.shape[0], _ptr(weight),
                                                   _ptr(bias), _ptr(pre), _ptr(y), _ptr(table), n_expert, int(rows_cap),
-                                                  in_feat, out_feat, dt, activation, _stream(x)))
+                                                  in_feat, out_feat, dt, activation, _ptr(ws),
+                                                  0 if ws is None else ws.numel(), _stream(x)))
     return y, pre
 
 
@@ -640,10 +652,11 @@ def linear_dgrad_dev(grad_y, weight, table, rows_cap, pre=None, activation=_lib.
             raise ValueError(f"pre must be [>= {rows_cap}, {in_feat}]")
     grad_x = torch.empty(rows_cap, in_feat, dtype=grad_y.dtype, device=grad_y.device)
     with torch.cuda.device(grad_y.device):
+        ws = _dev_workspace(out_feat, dt, grad_y.device)
         check(_lib.load().fmoe_linear_dgrad_dev(_ptr(grad_y), _ptr(weight),
                                                 _ptr(pre if activation != _lib.ACT_NONE else None), _ptr(grad_x),
                                                 _ptr(table), n_expert, int(rows_cap), in_feat, out_feat, dt, activation,
-                                                _stream(grad_y)))
+                                                _ptr(ws), 0 if ws is None else ws.numel(), _stream(grad_y)))
     return grad_x
 
 

@@ -380,6 +380,14 @@ int fmoe_segment_table_build(const int64_t *expert_count, int64_t n_expert,
  * feature sizes that are multiples of 16 bytes), else 0.  Host only. */
 int fmoe_linear_dev_supported(int64_t in_feat, int64_t out_feat, int dtype);
 
+/* Bytes of workspace with which the two row-ragged products below can split a
+ * last, partial round of tiles along the contraction (the host-count entry
+ * points keep such a workspace inside the library; here it is the caller's, so
+ * that nothing on this path allocates); 0 when a contraction of `contraction`
+ * elements is too short to be split at all.  workspace may always be NULL: the
+ * last round is then not split. */
+int64_t fmoe_linear_dev_workspace_bytes(int64_t contraction, int dtype);
+
 /* fmoe_linear_forward / fmoe_linear_act_forward over a device table:
  *   pre[seg_e] = x[seg_e] . w[e]^T + bias[e]  (stored when pre != NULL)
  *   y[seg_e]   = act(pre[seg_e])              (activation FMOE_ACT_NONE: y = pre)
@@ -394,7 +402,8 @@ int fmoe_linear_forward_dev(const void *x, const int64_t *x_row_index,
                             const void *w, const void *bias, void *pre, void *y,
                             const void *segment_table, int64_t n_expert,
                             int64_t rows_cap, int64_t in_feat, int64_t out_feat,
-                            int dtype, int activation, void *stream);
+                            int dtype, int activation, void *workspace,
+                            int64_t workspace_bytes, void *stream);
 
 /* Data gradient, as fmoe_linear_dact_backward (activation FMOE_ACT_NONE: the
  * plain data gradient of fmoe_linear_backward, pre ignored). */
@@ -402,6 +411,7 @@ int fmoe_linear_dgrad_dev(const void *grad_y, const void *w, const void *pre,
                           void *grad_x, const void *segment_table,
                           int64_t n_expert, int64_t rows_cap, int64_t in_feat,
                           int64_t out_feat, int dtype, int activation,
+                          void *workspace, int64_t workspace_bytes,
                           void *stream);
 
 /* Weight and bias gradient, as the grad_w / grad_b half of fmoe_linear_backward

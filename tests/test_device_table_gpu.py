@@ -185,3 +185,35 @@ def test_unsupported_shapes_are_refused(device):
         fmoe_native.linear_forward_dev(x[:4].contiguous(), w, None, table, 8)   # fewer rows than rows_cap
     with pytest.raises(ValueError):
         fmoe_native.linear_forward_dev(x, w, None, table[:10].contiguous(), 8)  # table too short
+
+
+@pytest.mark.parametrize("tile", ["256x256", "128x256"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,slots,e,fin,fout", [
+    (600, 700, 2, 4096, 520),     # forward: a short last round of deep tiles -> split along the contraction
+    (600, 600, 3, 520, 4096),     # data gradient: the same
+    (70000, 70000, 4, 3584, 264), # more than one round of tiles before the split tail
+])
+def test_split_tail_over_the_device_table(dtype, rows, slots, e, fin, fout, tile, device, monkeypatch):
+    """A last, partial round of tiles is split along the contraction by the workgroups themselves when the
+    segments come from a device table (the host does not know the tile count): same plan, same order of
+    the partial sums and so the same bits as the host-count launch, with and without the caller's workspace
+    (FMOE_DEV_SPLIT=0: no workspace, no split -- another order of the sums, equal within the tolerance)."""
+    monkeypatch.setenv("FMOE_GEMM_TILE", tile)
+    g = torch.Generator().manual_seed(rows + fin)
+    counts = ragged_counts(rows, e, g, 0)
+    x = torch.randn(slots, fin, generator=g).to(dtype).to(device)
+    w = (torch.randn(e, fout, fin, generator=g) / fin ** 0.5).to(dtype).to(device)
+    b = torch.randn(e, fout, generator=g).to(dtype).to(device)
+    gy = torch.randn(slots, fout, generator=g).to(dtype).to(device)
+    table = fmoe_native.segment_table(counts.to(device), slots)
+    y_host = fmoe_native.linear_forward(x, counts, w, b)
+    gx_host = fmoe_native.linear_backward(gy, x, counts, w, b)[0]
+    for flag in ("1", "0"):
+        monkeypatch.setenv("FMOE_DEV_SPLIT", flag)
+        y, _ = fmoe_native.linear_forward_dev(x, w, b, table, slots)
+        gx = fmoe_native.linear_dgrad_dev(gy, w, table, slots)
+        if flag == "1":
+            assert torch.equal(y[:rows], y_host[:rows]) and torch.equal(gx[:rows], gx_host[:rows])
+        else:
+            assert rel_err(y[:rows], y_host[:rows]) <= TOL[dtype] and rel_err(gx[:rows], gx_host[:rows]) <= TOL[dtype]
