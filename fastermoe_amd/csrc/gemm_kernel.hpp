@@ -1131,27 +1131,34 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(float *ws, int k_spli
     base[0] = sum;
 }
 
-// The same for a launch over a device table: sized for the most tail tiles there can be, every
-// thread works out from the table's tile count whether (and how) the tail was split.
+// The same for a launch over a device table, sized for the most tail tiles there can be: kPerTile
+// workgroups per tile, each adding up its share of the tile in steps of 256 vectors; a workgroup
+// works out from the table's tile count whether (and how) the tail was split and leaves at once
+// when its tile does not exist.
+constexpr int kReducePerTile = 8;
 template <int kMaxSplit>
 __global__ __launch_bounds__(256) void split_reduce_dev_kernel(float *ws, const int32_t *__restrict__ dev_tab, int tiles_index,
                                                                int tiles_n, int n_slabs, int cus, int64_t tile_vecs) {
     typedef float f32x4 __attribute__((ext_vector_type(4)));
-    const int total = dev_tab[tiles_index] * tiles_n;
+    typedef const int32_t __attribute__((address_space(4))) *DevTab;
+    const int total = ((DevTab)(uintptr_t)dev_tab)[tiles_index] * tiles_n;
     const TailSplit ts = plan_tail_split(total, n_slabs, cus);
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t tile = i / tile_vecs, v = i - tile * tile_vecs;
+    const int tile = blockIdx.x / kReducePerTile, share = blockIdx.x % kReducePerTile;
     if (ts.k_split == 1 || tile >= total - ts.main_tiles) return;
-    f32x4 *base = (f32x4 *)ws + tile * ts.k_split * tile_vecs + v;
-    f32x4 part[kMaxSplit];
+    const int64_t per_share = (tile_vecs + kReducePerTile - 1) / kReducePerTile;
+    const int64_t v_end = (share + 1) * per_share < tile_vecs ? (share + 1) * per_share : tile_vecs;
+    for (int64_t v = share * per_share + threadIdx.x; v < v_end; v += 256) {
+        f32x4 *base = (f32x4 *)ws + (int64_t)tile * ts.k_split * tile_vecs + v;
+        f32x4 part[kMaxSplit];
 #pragma unroll
-    for (int p = 0; p < kMaxSplit; ++p)
-        if (p < ts.k_split) part[p] = __builtin_nontemporal_load(base + (int64_t)p * tile_vecs);
-    f32x4 sum = part[0];
+        for (int p = 0; p < kMaxSplit; ++p)
+            if (p < ts.k_split) part[p] = __builtin_nontemporal_load(base + (int64_t)p * tile_vecs);
+        f32x4 sum = part[0];
 #pragma unroll
-    for (int p = 1; p < kMaxSplit; ++p)
-        if (p < ts.k_split) sum += part[p];
-    base[0] = sum;
+        for (int p = 1; p < kMaxSplit; ++p)
+            if (p < ts.k_split) sum += part[p];
+        base[0] = sum;
+    }
 }
 
 // Host-side services of grouped_gemm.hip: compute units of the current device, and a per-stream
@@ -1243,7 +1250,7 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
         constexpr int BKE = kSlabBytes / (int)sizeof(T);
         const int max_tail = prm.dev_cus / 2;
         const int64_t tile_vecs = (int64_t)BM * BN / 4;
-        split_reduce_dev_kernel<kMaxSplit><<<(unsigned)((tile_vecs * max_tail + 255) / 256), 256, 0, stream>>>(
+        split_reduce_dev_kernel<kMaxSplit><<<(unsigned)(max_tail * kReducePerTile), 256, 0, stream>>>(
             prm.split_ws, prm.dev_tab, BM == 256 ? segtab::kTiles256 : segtab::kTiles128, prm.tiles_n,
             (prm.k_extent + BKE - 1) / BKE, prm.dev_cus, tile_vecs);
         FMOE_LAUNCH_CHECK();
