@@ -26,7 +26,7 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wall", "-Wno-
 # extra -D switches for experiments, e.g. FMOE_EXTRA_FLAGS="-DFMOE_X=1"
 FLAGS += os.environ.get("FMOE_EXTRA_FLAGS", "").split()
 
-PLAIN_UNITS = ["error.cpp", "profile.cpp", "routing.hip", "segment_table.hip", "permute.hip", "combine.hip", "grouped_gemm.hip", "pipeline.hip"]
+PLAIN_UNITS = ["error.cpp", "profile.cpp", "routing.hip", "segment_table.hip", "permute.hip", "combine.hip", "grouped_gemm.hip", "gemm_any.hip", "pipeline.hip"]
 GEMM_TYPES = {0: "f32", 1: "bf16", 2: "f16"}
 GEMM_PRODUCTS = {0: "fwd", 1: "dgrad", 2: "wgrad"}
 

@@ -29,7 +29,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kWavesN = 2;
 constexpr int waves_m_of(int bn) { return bn == 128 ? 2 : 4; }
 constexpr int threads_of(int bn) { return 64 * waves_m_of(bn) * kWavesN; }
-constexpr int kThreads = threads_of(256);  // the any-shape kernels' workgroup size
+constexpr int kThreads = threads_of(256);  // workgroup size of the stand-alone bias-gradient kernel
 // The first kLoadWaves waves of a workgroup request the slabs.  The SIMD issues from its
 // oldest wave first, so with two waves per SIMD the younger one falls behind; leaving the
 // loads (which can block at a full load queue) to the older waves evens the two out.
@@ -1312,5 +1312,8 @@ FMOE_DECLARE_MFMA(launch_mfma_f16_wgrad);
 FMOE_DECLARE_MFMA(launch_mfma_f32_fwd);
 FMOE_DECLARE_MFMA(launch_mfma_f32_dgrad);
 FMOE_DECLARE_MFMA(launch_mfma_f32_wgrad);
+// double precision, and any type with feature sizes or pointers off the 16-byte grid; all three products
+// (0 forward, 1 data gradient, 2 weight gradient): gemm_any.hip
+int launch_mfma_any(gemm::GemmParams &prm, int dtype, int product, int epilogue, hipStream_t stream);
 
 }  // namespace fmoe

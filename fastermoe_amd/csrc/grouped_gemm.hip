@@ -11,8 +11,8 @@
 //   wgrad    dW_e    = dY[seg]^T . X[seg]  contraction ragged (the segment)
 //
 // This file holds the host side: segment tables, launch plans per product and per
-// chunk, the any-shape fallback kernel (feature sizes that are not a multiple of 16
-// bytes, fp64) and the stand-alone bias-gradient kernel that fallback needs.  The MFMA
+// chunk and the stand-alone bias-gradient kernel that the any-shape kernel of gemm_any.hip (feature
+// sizes that are not a multiple of 16 bytes, fp64) needs.  The MFMA
 // kernel itself (tiling, LDS layouts, software pipeline, epilogues) is in
 // gemm_kernel.hpp and is instantiated once per element type and product by
 // gemm_inst.hip.
@@ -29,47 +29,6 @@
 namespace fmoe {
 using namespace gemm;
 namespace {
-
-// ---- any-shape fallback (odd feature sizes, fp64): one thread per C element ----
-template <typename T, typename Acc, int RAGGED, int PSHAPE>
-__global__ __launch_bounds__(kThreads) void grouped_gemm_plain_kernel(const GemmParams prm) {
-    const int ei = blockIdx.z;
-    const int expert = prm.tab.first_expert + ei;
-    const int seg_lo = prm.tab.seg[ei], seg_hi = prm.tab.seg[ei + 1];
-    const int col = blockIdx.x * 16 + (threadIdx.x & 15);
-    const int rows = (RAGGED == kRaggedRows) ? seg_hi - seg_lo : prm.n_rows;
-    const T *bias = prm.bias ? (const T *)prm.bias + (int64_t)expert * prm.bias_expert_stride : nullptr;
-    const bool accumulate = (RAGGED == kRaggedK) && prm.accumulate_first && ei == 0;
-    if (col >= prm.n_cols) return;
-    for (int row = blockIdx.y * 16 + (threadIdx.x >> 4); row < rows; row += gridDim.y * 16) {
-        Acc acc = 0;
-        int64_t c_off;
-        if (RAGGED == kRaggedRows) {
-            const T *q = (const T *)prm.Q + (int64_t)(seg_lo + row) * prm.ldq;
-            const T *p = (const T *)prm.P + (int64_t)expert * prm.p_expert_stride;
-            for (int k = 0; k < prm.k_extent; ++k) {
-                const Acc pv = (PSHAPE == kKC) ? (Acc)p[(int64_t)col * prm.ldp + k] : (Acc)p[(int64_t)k * prm.ldp + col];
-                acc += (Acc)q[k] * pv;
-            }
-            c_off = (int64_t)(seg_lo + row) * prm.ldc + col;
-        } else {
-            const T *q = (const T *)prm.Q + (int64_t)seg_lo * prm.ldq + row;
-            const T *p = (const T *)prm.P + (int64_t)seg_lo * prm.ldp + col;
-            for (int k = 0; k < seg_hi - seg_lo; ++k) acc += (Acc)q[(int64_t)k * prm.ldq] * (Acc)p[(int64_t)k * prm.ldp];
-            c_off = (int64_t)expert * prm.c_expert_stride + (int64_t)row * prm.ldc + col;
-        }
-        T *dst = (T *)prm.C + c_off;
-        if (bias) acc += (Acc)bias[col];
-        if (prm.epilogue == kEpiBiasAct) {
-            if (prm.aux) ((T *)prm.aux)[c_off] = (T)acc;
-            acc = (Acc)apply_act<false>((float)acc, prm.activation);
-        } else if (prm.epilogue == kEpiDAct) {
-            acc *= (Acc)act_grad<false>((float)((const T *)prm.aux)[c_off], prm.activation);
-        }
-        if (accumulate) acc += (Acc)*dst;
-        *dst = (T)acc;
-    }
-}
 
 // ---- bias gradient: column sums per expert segment ---------------------------------
 // Thread (c, g) adds rows g, g+4, ... of column c in order; the four partial sums
@@ -238,24 +197,6 @@ template <typename T> bool fast_ok(std::initializer_list<const void *> ptrs, std
     return true;
 }
 
-template <typename T, typename Acc, int RG, int PS>
-int launch_plain(GemmParams &prm, int epi, hipStream_t stream) {
-    prm.epilogue = epi;
-    int max_rows = 0;
-    if (RG == kRaggedRows) {
-        for (int i = 0; i < prm.tab.n; ++i) max_rows = std::max(max_rows, prm.tab.seg[i + 1] - prm.tab.seg[i]);
-    } else {
-        max_rows = prm.n_rows;
-    }
-    if (max_rows == 0 || prm.n_cols == 0) return FMOE_OK;
-    dim3 grid((unsigned)ceil_div(prm.n_cols, 16), (unsigned)std::min<int64_t>(ceil_div(max_rows, 16), 1024),
-              (unsigned)prm.tab.n);
-    ProfileScope prof(prm.profile_class, prm.profile_work, stream);
-    grouped_gemm_plain_kernel<T, Acc, RG, PS><<<grid, kThreads, 0, stream>>>(prm);
-    FMOE_LAUNCH_CHECK();
-    return FMOE_OK;
-}
-
 enum Product { kFwd = 0, kDgrad = 1, kWgrad = 2 };
 
 struct SplitBuffer {
@@ -270,17 +211,8 @@ int g_compute_units[16] = {};
 
 template <int PRODUCT>
 int dispatch(GemmParams &prm, int dtype, int epi, bool fast, hipStream_t stream) {
-    constexpr int RG = PRODUCT == kWgrad ? kRaggedK : kRaggedRows;
-    constexpr int PS = PRODUCT == kFwd ? kKC : kMC;
-    if (!fast || dtype == FMOE_F64) {
-        switch (dtype) {
-            case FMOE_BF16: return launch_plain<__bf16, float, RG, PS>(prm, epi, stream);
-            case FMOE_F16: return launch_plain<_Float16, float, RG, PS>(prm, epi, stream);
-            case FMOE_F32: return launch_plain<float, float, RG, PS>(prm, epi, stream);
-            case FMOE_F64: return launch_plain<double, double, RG, PS>(prm, epi, stream);
-        }
-        return fail(FMOE_EINVAL, "unknown dtype %d", dtype);
-    }
+    // double precision, and shapes off the 16-byte grid: the element-checked kernel of gemm_any.hip
+    if (!fast || dtype == FMOE_F64) return launch_mfma_any(prm, dtype, PRODUCT, epi, stream);
     switch (dtype * 3 + PRODUCT) {
         case FMOE_BF16 * 3 + kFwd: return launch_mfma_bf16_fwd(prm, epi, stream);
         case FMOE_BF16 * 3 + kDgrad: return launch_mfma_bf16_dgrad(prm, epi, stream);
