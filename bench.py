@@ -39,8 +39,8 @@ PEAK = {"bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
 # HBM-side bytes per launch of the grouped GEMM at config 4 (rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
 # what the same counter reads for a copy kernel of known size: 1.984 and 1.000); measured offline, not in this
 # script -- the counters need their own profiler runs.  Per class the mean over its launches of a step: forward
-# (2.99 + 0.93 and 2.98 + 0.13 GB), data-grad (3.44 + 0.46 and 2.98 + 0.13 GB), weight-grad (16.89 + 0.94 GB, all rows).
-TRAFFIC_BYTES = {"config4": {"gemm_fwd": 3.52e9, "gemm_dgrad": 3.51e9, "gemm_wgrad": 17.8e9}}
+# (2.96 + 0.93 and 2.95 + 0.13 GB), data-grad (3.41 + 0.47 and 2.95 + 0.13 GB), weight-grad (17.65 + 0.94 GB, all rows).
+TRAFFIC_BYTES = {"config4": {"gemm_fwd": 3.49e9, "gemm_dgrad": 3.48e9, "gemm_wgrad": 18.6e9}}
 TRAFFIC_SOURCE = "profiles/grouped_gemm_bf16_config4_hbm_traffic.md (rocprofv3 --pmc runs, not this run)"
 HBM_PEAK_GBS = 8000.0
 
