@@ -230,36 +230,40 @@ inline void set_row_index_divisor(GemmParams &prm, int64_t divisor) {
 }
 
 // How the tiles of a ragged-rows launch are spread over the chip.  One workgroup occupies a
-// compute unit, so `total` tiles run in total / cus rounds and a last, partial round costs as
-// much as a whole one.  When that last round fills at most half the chip, its tiles are split
-// along the contraction into k_split parts (as many as fit the idle units, at most 8, at
-// least 16 slabs each) -- provided that shortens the round by more than the partial sums' round
-// trip through memory costs.  Evaluated on the host for launches over host counts and by every
-// workgroup for launches over a device table (where only the device knows the tile count).
+// compute unit (two 128 x 128 workgroups share one, and then share its matrix pipe), so `total`
+// tiles run in total / cus rounds and a last, partial round costs as much as a whole one.  When
+// that last round fills at most half the chip, its tiles are split along the contraction into
+// k_split parts (as many as fit the idle units, at most 8, at least 16 slabs each) -- provided
+// that shortens the round by more than the partial sums' round trip through memory costs.
+// slab_weight is the matrix-pipe time of a slab in units of a 16-bit slab's (2 for fp32: the same
+// 128 bytes per row hold half the elements, each at a quarter of the rate).  Evaluated on the host
+// for launches over host counts and by every workgroup for launches over a device table (where
+// only the device knows the tile count).
 constexpr int kMaxSplit = 8;
 struct TailSplit {
     int main_tiles, k_split, split_slabs;
 };
-__host__ __device__ inline TailSplit plan_tail_split(int total, int n_slabs, int cus) {
+__host__ __device__ inline TailSplit plan_tail_split(int total, int n_slabs, int cus, int slab_weight = 1) {
     TailSplit p{total, 1, n_slabs};
     const int tail = total % cus;
     if (tail == 0 || tail * 2 > cus) return p;
     int f = cus / tail < kMaxSplit ? cus / tail : kMaxSplit;
-    f = n_slabs / 16 < f ? n_slabs / 16 : f;
+    f = n_slabs * slab_weight / 16 < f ? n_slabs * slab_weight / 16 : f;
     if (f < 2) return p;
     const int per_part = (n_slabs + f - 1) / f;
-    // the reduction and the second launch cost about as much as 40 slabs of one tile
-    if (n_slabs - per_part < 40) return p;
+    // the reduction and the second launch cost about as much as 40 (16-bit) slabs of one tile
+    if ((n_slabs - per_part) * slab_weight < 40) return p;
     p.split_slabs = per_part;
     p.k_split = (n_slabs + p.split_slabs - 1) / p.split_slabs;  // no empty part
     p.main_tiles = total - tail;
     return p;
 }
 // whether any tile count at all makes plan_tail_split split a contraction of n_slabs slabs
-inline bool tail_split_possible(int n_slabs) {
-    const int f = n_slabs / 16 < kMaxSplit ? n_slabs / 16 : kMaxSplit;
-    return f >= 2 && n_slabs - (n_slabs + f - 1) / f >= 40;
+inline bool tail_split_possible(int n_slabs, int slab_weight = 1) {
+    const int f = n_slabs * slab_weight / 16 < kMaxSplit ? n_slabs * slab_weight / 16 : kMaxSplit;
+    return f >= 2 && (n_slabs - (n_slabs + f - 1) / f) * slab_weight >= 40;
 }
+template <typename T> constexpr int slab_weight_of() { return sizeof(T) == 4 ? 2 : 1; }
 
 // KC slabs: 16-byte chunk c of row r is stored at chunk c ^ swz(r).
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
                 tm_total = dtab[BM == 256 ? segtab::kTiles256 : segtab::kTiles128];
                 main_tiles = total_tiles = tm_total * prm.tiles_n;
                 if (prm.dev_cus > 0) {
-                    const TailSplit ts = plan_tail_split(total_tiles, (prm.k_extent + BKE - 1) / BKE, prm.dev_cus);
+                    const TailSplit ts = plan_tail_split(total_tiles, (prm.k_extent + BKE - 1) / BKE, prm.dev_cus, slab_weight_of<T>());
                     main_tiles = ts.main_tiles;
                     k_split = ts.k_split;
                     split_slabs = ts.split_slabs;
@@ -1138,11 +1142,12 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(float *ws, int k_spli
 constexpr int kReducePerTile = 8;
 template <int kMaxSplit>
 __global__ __launch_bounds__(256) void split_reduce_dev_kernel(float *ws, const int32_t *__restrict__ dev_tab, int tiles_index,
-                                                               int tiles_n, int n_slabs, int cus, int64_t tile_vecs) {
+                                                               int tiles_n, int n_slabs, int cus, int slab_weight,
+                                                               int64_t tile_vecs) {
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     typedef const int32_t __attribute__((address_space(4))) *DevTab;
     const int total = ((DevTab)(uintptr_t)dev_tab)[tiles_index] * tiles_n;
-    const TailSplit ts = plan_tail_split(total, n_slabs, cus);
+    const TailSplit ts = plan_tail_split(total, n_slabs, cus, slab_weight);
     const int tile = blockIdx.x / kReducePerTile, share = blockIdx.x % kReducePerTile;
     if (ts.k_split == 1 || tile >= total - ts.main_tiles) return;
     const int64_t per_share = (tile_vecs + kReducePerTile - 1) / kReducePerTile;
@@ -1199,19 +1204,18 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
     if (RG == kRaggedRows) {
         constexpr int BKE = kSlabBytes / (int)sizeof(T);
         const int n_slabs = (prm.k_extent + BKE - 1) / BKE;
-        // (two 128 x 128 workgroups share a compute unit: their launches are not split)
+        constexpr int kWeight = slab_weight_of<T>();
         if (prm.dev_tab != nullptr) {
             // the host does not know the tile count: with a workspace from the caller, every workgroup plans the
             // split itself, and the launch is sized for the most parts there can be (one per compute unit)
             prm.dev_cus = 0;
-            if (BN == 256 && prm.dev_split_ws != nullptr && tail_split_possible(n_slabs)) {
+            if (prm.dev_split_ws != nullptr && tail_split_possible(n_slabs, kWeight)) {
                 prm.dev_cus = device_compute_units();
                 prm.split_ws = prm.dev_split_ws;
             }
             grid64 = ((int64_t)prm.total_tiles + 7) / 8 * 8 + prm.dev_cus;
         } else {
-            const TailSplit ts = BN == 256 ? plan_tail_split(prm.total_tiles, n_slabs, device_compute_units())
-                                           : TailSplit{prm.total_tiles, 1, n_slabs};
+            const TailSplit ts = plan_tail_split(prm.total_tiles, n_slabs, device_compute_units(), kWeight);
             if (ts.k_split > 1) {
                 const int tail = prm.total_tiles - ts.main_tiles;
                 float *ws = split_workspace(stream, (size_t)tail * ts.k_split * BM * BN * sizeof(float));
@@ -1252,7 +1256,7 @@ int launch_tiles(GemmParams &prm, hipStream_t stream) {
         const int64_t tile_vecs = (int64_t)BM * BN / 4;
         split_reduce_dev_kernel<kMaxSplit><<<(unsigned)(max_tail * kReducePerTile), 256, 0, stream>>>(
             prm.split_ws, prm.dev_tab, BM == 256 ? segtab::kTiles256 : segtab::kTiles128, prm.tiles_n,
-            (prm.k_extent + BKE - 1) / BKE, prm.dev_cus, tile_vecs);
+            (prm.k_extent + BKE - 1) / BKE, prm.dev_cus, slab_weight_of<T>(), tile_vecs);
         FMOE_LAUNCH_CHECK();
         prm.fixup = 1;
         kern<<<max_tail * kWavesM * kWavesN, 64, smem_wave_epi, stream>>>(prm);

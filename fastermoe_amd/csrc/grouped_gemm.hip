@@ -306,7 +306,7 @@ int64_t linear_dev_workspace_bytes(int64_t contraction, int dtype) {
     const int eb = dtype_bytes(dtype);
     if (eb == 0 || dtype == FMOE_F64 || contraction < 1) return 0;
     const int64_t per_slab = kSlabBytes / eb;
-    if (!tail_split_possible((int)std::min<int64_t>(ceil_div(contraction, per_slab), 1 << 24))) return 0;
+    if (!tail_split_possible((int)std::min<int64_t>(ceil_div(contraction, per_slab), 1 << 24), eb == 4 ? 2 : 1)) return 0;
     // one tile of fp32 accumulators per compute unit: a split never has more parts than that
     return (int64_t)device_compute_units() * 256 * 256 * (int64_t)sizeof(float);
 }
