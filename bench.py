@@ -256,7 +256,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", dest="other_configs", action="store_false",
                     help="skip the short runs of configurations 1, 2, 3 and 5 that follow the headline workload")
-    ap.add_argument("--profile-steps", type=int, default=3)
+    ap.add_argument("--profile-steps", type=lambda v: max(1, int(v)), default=3,
+                    help="steps run with the library's per-launch HIP-event brackets after the timed ones (at least 1)")
     ap.add_argument("--no-gate-linear", dest="gate_linear", action="store_false",
                     help="skip the second figure with the gate's linear layer inside the step")
     ap.add_argument("--fuse", choices=["auto", "on", "off"], default="auto",
