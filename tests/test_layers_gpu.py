@@ -1034,3 +1034,54 @@ def test_noisy_top_k_16_bit_against_float64(dtype, n, e, k, device):
     assert rel_err(gates, ref_gates) <= tol and rel_err(load, ref_load) <= 1e-4
     assert_close(clean.grad, c64.grad, tol, "grad_clean")
     assert_close(raw.grad, r64.grad, tol, "grad_raw")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ["one_token", "one_expert_takes_all", "all_dropped", "single_expert_layer",
+                                  "one_slot_survives", "more_experts_than_rows"])
+def test_device_table_path_at_extreme_routings(case, dtype, device):
+    """The layer's own unfused path (segment table built on the device, launches sized for an upper
+    bound of tiles) at the routings that stress that bound: a single token, every slot on one expert,
+    no surviving slot at all, a one-expert layer, a single surviving slot, and more experts than
+    rows.  Against the brute-force oracle (tests/moe.py:30-49 semantics: a dropped slot contributes a
+    zero row); experts without rows must come out with zero gradients."""
+    torch.manual_seed(91)
+    n, d, h, e, k = 37, 64, 96, 6, 2
+    if case == "one_token":
+        n = 1
+    if case == "single_expert_layer":
+        e, k = 1, 1
+    if case == "more_experts_than_rows":
+        n, e = 3, 40
+    moe = fmoe.FMoETransformerMLP(num_expert=e, d_model=d, d_hidden=h, top_k=k, activation=nn.GELU())
+    moe = moe.to(dtype).to(device)
+    x = torch.randn(n, d).to(dtype).to(device)
+    idx = torch.randint(0, e, (n, k), device=device)
+    if case == "one_expert_takes_all":
+        idx.fill_(e - 2)
+    elif case == "all_dropped":
+        idx.fill_(-1)
+    elif case == "one_slot_survives":
+        idx.fill_(-1)
+        idx[n // 2, 1] = 3
+    score = torch.rand(n, k, device=device).to(dtype)
+    x = x.clone().requires_grad_(True)
+    moe.gate.forward = lambda inp: (idx, score)
+    out = moe(x)
+    out.float().sum().backward()
+    ex = moe.experts
+    ref = omoe.moe_mlp_forward_backward(x, idx, score, ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias,
+                                        nn.GELU(), k, loss="sum")
+    tol = TOL[dtype]
+    got = {"out": out, "grad_inp": x.grad, "grad_w1": ex.htoh4.weight.grad, "grad_w2": ex.h4toh.weight.grad,
+           "grad_b1": ex.htoh4.bias.grad, "grad_b2": ex.h4toh.bias.grad}
+    counts = torch.bincount(idx[idx >= 0].view(-1).cpu(), minlength=e)
+    for name, val in got.items():
+        assert val is not None and torch.isfinite(val.float()).all(), name
+        want = ref[name] if ref[name] is not None else torch.zeros(val.shape, dtype=torch.float64)   # (no slot used it)
+        scale = max(want.abs().max().item(), 1.0)
+        assert (val.double().cpu() - want.double().cpu()).abs().max().item() <= tol * scale, name
+    for name in ("grad_w1", "grad_w2", "grad_b1", "grad_b2"):
+        for expert in range(e):
+            if counts[expert] == 0:
+                assert torch.count_nonzero(got[name][expert]) == 0, (name, expert)
