@@ -28,12 +28,12 @@ constexpr int kThreads64 = 256;
 
 __device__ __forceinline__ double act_f64(double x, int act) {
     if (act == FMOE_ACT_RELU) return x > 0.0 ? x : 0.0;
-    if (act == FMOE_ACT_GELU) return 0.5 * x * (1.0 + erf(x * 0.70710678118654752440));
+    if (act == FMOE_ACT_GELU || act == gemm::kActGeluErf) return 0.5 * x * (1.0 + erf(x * 0.70710678118654752440));
     return x;
 }
 __device__ __forceinline__ double act_grad_f64(double x, int act) {
     if (act == FMOE_ACT_RELU) return x > 0.0 ? 1.0 : 0.0;
-    if (act == FMOE_ACT_GELU)
+    if (act == FMOE_ACT_GELU || act == gemm::kActGeluErf)
         return 0.5 * (1.0 + erf(x * 0.70710678118654752440)) + x * 0.39894228040143267794 * exp(-0.5 * x * x);
     return 1.0;
 }

@@ -142,11 +142,15 @@ __device__ __forceinline__ float gelu_grad_16bit(float x) {
     return fmaf(x, 0.f, fmaf(xc, r, 0.5f));
 }
 
+// Activation code inside the kernels only: exact GELU with the erf formula whatever the element type
+// (FMOE_ACT_GELU takes the polynomials when the result is rounded to 16 bits).
+constexpr int kActGeluErf = 3;
+
 // kNarrow: the result is rounded to a 16-bit type
 template <bool kNarrow> __device__ __forceinline__ float apply_act(float x, int act) {
     if (act == FMOE_ACT_RELU) return x > 0.f ? x : 0.f;
-    if (act == FMOE_ACT_GELU) {
-        if (kNarrow) return fmaf(x, cdf_minus_half_16bit(x), 0.5f * x);
+    if (act == FMOE_ACT_GELU || act == kActGeluErf) {
+        if (kNarrow && act == FMOE_ACT_GELU) return fmaf(x, cdf_minus_half_16bit(x), 0.5f * x);
         return x * gelu_terms(x).cdf;
     }
     return x;
@@ -154,8 +158,8 @@ template <bool kNarrow> __device__ __forceinline__ float apply_act(float x, int 
 
 template <bool kNarrow> __device__ __forceinline__ float act_grad(float x, int act) {
     if (act == FMOE_ACT_RELU) return x > 0.f ? 1.f : 0.f;
-    if (act == FMOE_ACT_GELU) {
-        if (kNarrow) return gelu_grad_16bit(x);
+    if (act == FMOE_ACT_GELU || act == kActGeluErf) {
+        if (kNarrow && act == FMOE_ACT_GELU) return gelu_grad_16bit(x);
         const GeluTerms g = gelu_terms(x);
         return g.cdf + x * g.pdf;
     }
@@ -1099,6 +1103,8 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
     typedef std::integral_constant<int, FMOE_ACT_NONE> ActNone;
     auto by_activation = [&](auto auxreg_tag) {
         if (prm.activation == FMOE_ACT_GELU) run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{}, auxreg_tag);
+        else if (sizeof(T) == 2 && prm.activation == kActGeluErf) run_epilogue(std::integral_constant<int, kActGeluErf>{}, std::false_type{}, auxreg_tag);
+        else if (prm.activation == kActGeluErf) run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{}, auxreg_tag);
         else if (prm.activation == FMOE_ACT_RELU) run_epilogue(std::integral_constant<int, FMOE_ACT_RELU>{}, std::false_type{}, auxreg_tag);
         else run_epilogue(ActNone{}, std::false_type{}, auxreg_tag);
     };

@@ -104,6 +104,18 @@ TileShape pick_tile(int64_t tiles_256) {
     return tiles_256 >= 256 ? TileShape{128, 256} : TileShape{128, 128};
 }
 
+// The activation code the kernels see.  For results that are rounded to a 16-bit type GELU and its
+// derivative come from polynomials (gemm_kernel.hpp); FMOE_GELU_ERF=1 selects the erf formula of
+// the 32-bit path for them too (|error| <= 1.5e-7 instead of 4e-5 .. 1.4e-4, at about twice the
+// epilogue's arithmetic).
+int kernel_activation(int activation) {
+    if (activation == FMOE_ACT_GELU) {
+        const char *e = getenv("FMOE_GELU_ERF");
+        if (e && e[0] == '1') return gemm::kActGeluErf;
+    }
+    return activation;
+}
+
 // ragged rows: tiles_256 counts every expert's rows rounded up to whole 256-row tiles
 TileShape pick_rows_tile(const int64_t *counts, int64_t n_expert, int64_t row_lo, int64_t row_hi, int64_t n_cols) {
     int64_t start = 0, row_tiles = 0;
@@ -332,7 +344,7 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.bias_expert_stride = a.out_feat;
         prm.n_cols = (int)a.out_feat; prm.k_extent = (int)a.in_feat;
-        prm.activation = a.activation;
+        prm.activation = kernel_activation(a.activation);
         const int64_t ws_need = linear_dev_workspace_bytes(a.in_feat, a.dtype);
         if (a.dev_workspace != nullptr && ws_need > 0 && a.dev_workspace_bytes >= ws_need && aligned16(a.dev_workspace))
             prm.dev_split_ws = (float *)a.dev_workspace;
@@ -361,7 +373,7 @@ int grouped_linear_forward(const LinearForwardArgs &a, const int64_t *counts, in
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.bias_expert_stride = a.out_feat;
         prm.n_cols = (int)a.out_feat; prm.k_extent = (int)a.in_feat;
-        prm.activation = a.activation;
+        prm.activation = kernel_activation(a.activation);
         if (int rc = dispatch<kFwd>(prm, a.dtype, a.epilogue, fast, stream)) return rc;
     }
     return FMOE_OK;
@@ -384,7 +396,7 @@ int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts, int64_
         prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.n_cols = (int)a.in_feat; prm.k_extent = (int)a.out_feat;
-        prm.activation = a.activation;
+        prm.activation = kernel_activation(a.activation);
         const int64_t ws_need = linear_dev_workspace_bytes(a.out_feat, a.dtype);
         if (a.dev_workspace != nullptr && ws_need > 0 && a.dev_workspace_bytes >= ws_need && aligned16(a.dev_workspace))
             prm.dev_split_ws = (float *)a.dev_workspace;
@@ -409,7 +421,7 @@ int grouped_linear_dgrad(const LinearDgradArgs &a, const int64_t *counts, int64_
         prm.ldp = a.in_feat; prm.ldq = a.out_feat; prm.ldc = a.in_feat;
         prm.p_expert_stride = a.in_feat * a.out_feat;
         prm.n_cols = (int)a.in_feat; prm.k_extent = (int)a.out_feat;
-        prm.activation = a.activation;
+        prm.activation = kernel_activation(a.activation);
         if (int rc = dispatch<kDgrad>(prm, a.dtype, a.epilogue, fast, stream)) return rc;
     }
     return FMOE_OK;

@@ -598,13 +598,16 @@ def test_fused_many_experts_few_rows(chunks, device, monkeypatch):
     assert rel_err(results[1][2], ref["grad_w1"]) <= 1e-5
 
 
+@pytest.mark.parametrize("erf", ["0", "1"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-def test_fused_gelu_epilogue_accuracy(dtype, device):
+def test_fused_gelu_epilogue_accuracy(dtype, erf, device, monkeypatch):
     """The activation computed in the GEMM epilogue against torch's exact (erf) GELU of the
     saved pre-activation, over pre-activations from -9 to 9: within one rounding step of the
     element type (relative), plus 1e-4 absolute for the far negative tail where GELU -> 0;
-    and the derivative used by the backward against autograd's."""
+    and the derivative used by the backward against autograd's.  Both forms of the 16-bit
+    epilogues: the polynomials, and the erf formula that FMOE_GELU_ERF=1 selects."""
     from fastermoe_amd import _lib, fmoe_native
+    monkeypatch.setenv("FMOE_GELU_ERF", erf)
     n, d, h = 512, 64, 256
     x = torch.randn(n, d, device=device).to(dtype)
     w1 = (torch.randn(1, h, d, device=device) * 0.4).to(dtype)      # pre-activations ~ N(0, 3.2^2)
