@@ -422,8 +422,10 @@ int fmoe_linear_wgrad_dev(const void *grad_y, const void *x, void *grad_w,
                           int64_t out_feat, int dtype, void *stream);
 
 /* How a forward / data-grad launch of `total_tiles` output tiles (256 x 256, or
- * 128 x 256 for small launches) with `contraction_slabs` slabs of 128
- * contraction bytes is spread over `compute_units` (0: the current device's):
+ * 128 x 256 / 128 x 128 for small launches) of a 16-bit element type with
+ * `contraction_slabs` slabs of 128 contraction bytes (fp32 launches count
+ * every slab twice in the plan's thresholds: half the elements at a quarter
+ * of the rate) is spread over `compute_units` (0: the current device's):
  * plan_host[0] tiles are computed whole, one workgroup each; the rest -- the
  * last, partial round of the chip when it fills at most half of it -- are
  * split along the contraction into plan_host[1] parts of plan_host[2] slabs,
