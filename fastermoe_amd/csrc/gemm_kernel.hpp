@@ -1102,9 +1102,16 @@ __global__ __launch_bounds__(threads_of(BN)) void grouped_gemm_kernel(const Gemm
     };
     typedef std::integral_constant<int, FMOE_ACT_NONE> ActNone;
     auto by_activation = [&](auto auxreg_tag) {
-        if (prm.activation == FMOE_ACT_GELU) run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{}, auxreg_tag);
-        else if (sizeof(T) == 2 && prm.activation == kActGeluErf) run_epilogue(std::integral_constant<int, kActGeluErf>{}, std::false_type{}, auxreg_tag);
-        else if (prm.activation == kActGeluErf) run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{}, auxreg_tag);
+        // (every instantiation is called from one place only, so that it is inlined)
+        if constexpr (sizeof(T) == 2) {
+            if (prm.activation == kActGeluErf) {
+                run_epilogue(std::integral_constant<int, kActGeluErf>{}, std::false_type{}, auxreg_tag);
+                return;
+            }
+        }
+        // (a 32-bit type computes GELU with the erf formula anyway)
+        if (prm.activation == FMOE_ACT_GELU || prm.activation == kActGeluErf)
+            run_epilogue(std::integral_constant<int, FMOE_ACT_GELU>{}, std::false_type{}, auxreg_tag);
         else if (prm.activation == FMOE_ACT_RELU) run_epilogue(std::integral_constant<int, FMOE_ACT_RELU>{}, std::false_type{}, auxreg_tag);
         else run_epilogue(ActNone{}, std::false_type{}, auxreg_tag);
     };
